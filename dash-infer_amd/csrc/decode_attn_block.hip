@@ -117,7 +117,7 @@ __device__ __forceinline__ AbShare ab_share(const GemvArgs& g, int bid, int NB, 
 
 // the share is requested in the order the stand-alone kernel streams it, slots [J0, J1) per call (the cursor carries on).  Slots
 // beyond the share re-read the head of the matrix: every asm load is unconditional, so no register of the ring is defined on one
-// path only (a phi on an asm output may be resolved by a copy BEFORE the data has landed: tools/audit_asm_loads.py)
+// path only (a phi on an asm output may be resolved by a copy BEFORE the data has landed)
 struct AbCursor {
   const char* wtile;
   const char* stile;
@@ -359,7 +359,7 @@ __global__ __launch_bounds__(AB_THREADS) void decode_attn_block_kernel(const Att
 #pragma unroll
   for (int j = 0; j < 2; ++j) {
     // (both batches unconditionally, indices clamped: a batch defined on one path only is a phi, and the compiler resolves a phi on
-    // an asm load's registers with copies wherever it likes -- before the wait: tools/audit_asm_loads.py)
+    // an asm load's registers with copies wherever it likes -- before the wait)
     const uint32_t i = (uint32_t)min(j * AB_THREADS + tid, nvec_q - 1);
     stream_load_plain_b128(ev[2 * j], q.x, i * 32u);
     stream_load_plain_b128(ev[2 * j + 1], q.x, i * 32u + 16u);

@@ -260,7 +260,7 @@ __device__ __forceinline__ void gemv_stream_body(const GemvArgs& a, const int bi
   // `ev` / `eg` hold ONLY the batch issued here, ahead of the ring fill (row 0, vectors 0 ..): written by this asm, read after
   // the wait in the prologue, never assigned again.  (They used to be re-loaded for the later rows: two definitions make a
   // phi, the compiler resolves a phi with register copies wherever it likes -- it put them BEFORE the wait, and row 0 of a
-  // batch was now and then read before it had landed.  tools/audit_asm_loads.py checks the build for this.)
+  // batch was now and then read before it had landed.)
   // Every later batch (rows > 0, rows longer than one batch) goes through fetch_batch into registers of its own.
   const int Kp = a.KT * KTILE;  // == K (host contract)
   const int nvec = Kp >> 3;
@@ -705,7 +705,7 @@ __device__ __forceinline__ void gemv_stream_body(const GemvArgs& a, const int bi
   for (; c < total; c += D) {
 #pragma unroll
     for (int j = 0; j < D; ++j) {
-      if (c + j >= total) break;  // (a break, not a guard: no path consumes slot j + 1 without slot j -- tools/audit_asm_loads.py)
+      if (c + j >= total) break;  // (a break, not a guard: no path consumes slot j + 1 without slot j)
       stream_wait<(D - 1) * LPC>();
       stream_landed(wb[j], sb[j]);
       DIHIP_GEMV_CONSUME(j);

@@ -18,7 +18,7 @@
 //
 // (Until round 2 the quantised caches, and the 16-bit cache before its matrix-core form existed, went through a VALU
 // kernel with one query head per wave that did all of it in one launch: 22 - 325 spilled VGPRs depending on the heads per
-// group (profiles/r01j_kernel_resources.txt).  It is gone; the append launch costs one kernel boundary.)
+// group.  It is gone; the append launch costs one kernel boundary.)
 //
 // No inter-workgroup communication, no host work per step: sequence lengths are read on the device.
 #include <algorithm>
