@@ -1,0 +1,277 @@
+// seq_linear.hip -- dihip_linear: y = epilogue(x . W^T + bias) for row-major [N, K] weights as checkpoints store them,
+// grouped (block-diagonal / per-head) forms included.  Three kernels:
+//   linear_tile_kernel   every product and sum in f32, k ascending (DIHIP_MATH_F32; also any operand type / odd shape)
+//   linear_mfma_kernel   bf16 operands on the 16x16x32 matrix-core tiles, 128 x 128 x 32 block tiles, f32 accumulation
+//   linear_skinny_kernel up to 4 rows at a time against a streamed weight (decode): one wave per 4 weight rows
+// An output element is computed by one thread (or one MFMA column) over k in a fixed order: it does not depend on T.
+#include "seq_common.h"
+
+namespace dihip {
+namespace {
+
+struct LinArgs {
+  const void* x; long ldx, xg; int xgroups;
+  const void* w; const void* bias;
+  void* y; long ldy, yg;
+  const float* mul; long ldm;
+  int T, N, K, act, act_lo, act_hi, ydt, round_ops;
+};
+
+__device__ __forceinline__ void lin_epilogue(const LinArgs& a, int g, int t, int n, float v, int wdt) {
+  if (a.bias) v += ld_any(a.bias, (size_t)g * a.N + n, wdt);
+  const int col = g * a.N + n;
+  if (col >= a.act_lo && col < a.act_hi) v = apply_act(v, a.act);
+  const size_t o = (size_t)t * a.ldy + (size_t)g * a.yg + n;
+  if (a.mul) v *= a.mul[(size_t)t * a.ldm + (size_t)g * a.yg + n];
+  st_any(a.y, o, a.ydt, v);
+}
+
+// ------------------------------------------------------------------------------------------ exact f32 tile kernel
+template <int XT, int WT>
+__global__ __launch_bounds__(256) void linear_tile_kernel(LinArgs a) {
+  __shared__ float xs[16][68];
+  __shared__ float ws[16][68];
+  const int tid = threadIdx.x, tx = tid & 15, ty = tid >> 4;
+  const int g = blockIdx.z, m0 = blockIdx.y * 64, n0 = blockIdx.x * 64;
+  const size_t xoff = (size_t)(g % a.xgroups) * a.xg;
+  const size_t wbase = (size_t)g * a.N * a.K;
+  float acc[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[i][j] = 0.f;
+  for (int k0 = 0; k0 < a.K; k0 += 16) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int idx = tid + 256 * j, r = idx >> 4, kk = idx & 15;
+      float xv = 0.f, wv = 0.f;
+      if (k0 + kk < a.K) {
+        if (m0 + r < a.T) xv = load_ft<XT>(a.x, (size_t)(m0 + r) * a.ldx + xoff + k0 + kk);
+        if (n0 + r < a.N) wv = load_ft<WT>(a.w, wbase + (size_t)(n0 + r) * a.K + k0 + kk);
+      }
+      if (a.round_ops) { xv = ft_round<DIHIP_BF16>(xv); wv = ft_round<DIHIP_BF16>(wv); }
+      xs[kk][r] = xv;
+      ws[kk][r] = wv;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int kk = 0; kk < 16; ++kk) {
+      const f32x4_t av = *reinterpret_cast<const f32x4_t*>(&xs[kk][ty * 4]);
+      const f32x4_t bv = *reinterpret_cast<const f32x4_t*>(&ws[kk][tx * 4]);
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = __builtin_fmaf(av[i], bv[j], acc[i][j]);
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int t = m0 + ty * 4 + i;
+    if (t >= a.T) continue;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int n = n0 + tx * 4 + j;
+      if (n < a.N) lin_epilogue(a, g, t, n, acc[i][j], WT);
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------------------ bf16 matrix-core kernel
+__device__ __forceinline__ f32x4_t mfma_bf16(const u32x4_t& a, const u32x4_t& b, const f32x4_t& c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
+}
+
+// 8 consecutive k of one row as packed bf16; VEC: the 8 are in range and 16-byte aligned (host-checked), else guarded
+template <int XT, bool VEC>
+__device__ __forceinline__ u32x4_t load8_bf16(const void* p, size_t i, int kleft, bool row_ok) {
+  u32x4_t r = {0u, 0u, 0u, 0u};
+  if (!row_ok || kleft <= 0) return r;
+  if constexpr (VEC) {
+    if constexpr (XT == DIHIP_F32) {
+      const f32x4_t lo = *reinterpret_cast<const f32x4_t*>((const float*)p + i);
+      const f32x4_t hi = *reinterpret_cast<const f32x4_t*>((const float*)p + i + 4);
+      r[0] = pack_bf16x2(lo[0], lo[1]); r[1] = pack_bf16x2(lo[2], lo[3]);
+      r[2] = pack_bf16x2(hi[0], hi[1]); r[3] = pack_bf16x2(hi[2], hi[3]);
+    } else {
+      r = *reinterpret_cast<const u32x4_t*>((const uint16_t*)p + i);
+    }
+  } else {
+    uint32_t e[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) e[j] = j < kleft ? f32_to_bf16_bits(load_ft<XT>(p, i + j)) : 0u;
+    r[0] = e[0] | (e[1] << 16); r[1] = e[2] | (e[3] << 16); r[2] = e[4] | (e[5] << 16); r[3] = e[6] | (e[7] << 16);
+  }
+  return r;
+}
+
+template <int XT, bool VEC>
+__global__ __launch_bounds__(256) void linear_mfma_kernel(LinArgs a) {
+  constexpr int LD = 40;  // bf16 elements per LDS row: 32 + 8 of padding (80 bytes: 16-byte aligned fragments)
+  __shared__ __attribute__((aligned(16))) uint16_t As[128 * LD];
+  __shared__ __attribute__((aligned(16))) uint16_t Bs[128 * LD];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int g = blockIdx.z, m0 = blockIdx.y * 128, n0 = blockIdx.x * 128;
+  const size_t xoff = (size_t)(g % a.xgroups) * a.xg;
+  const size_t wbase = (size_t)g * a.N * a.K;
+  const f32x4_t z4 = {0.f, 0.f, 0.f, 0.f};
+  f32x4_t acc[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[i][j] = z4;
+  u32x4_t ra[2], rb[2];
+  auto fetch = [&](int k0) {
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int u = tid + 256 * j, r = u >> 2, k = k0 + (u & 3) * 8;
+      ra[j] = load8_bf16<XT, VEC>(a.x, (size_t)(m0 + r) * a.ldx + xoff + k, a.K - k, m0 + r < a.T);
+      rb[j] = load8_bf16<DIHIP_BF16, VEC>(a.w, wbase + (size_t)(n0 + r) * a.K + k, a.K - k, n0 + r < a.N);
+    }
+  };
+  fetch(0);
+  for (int k0 = 0; k0 < a.K; k0 += 32) {
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int u = tid + 256 * j, r = u >> 2, kq = (u & 3) * 8;
+      *reinterpret_cast<u32x4_t*>(&As[r * LD + kq]) = ra[j];
+      *reinterpret_cast<u32x4_t*>(&Bs[r * LD + kq]) = rb[j];
+    }
+    __syncthreads();
+    if (k0 + 32 < a.K) fetch(k0 + 32);
+    u32x4_t af[4], bf[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      af[i] = *reinterpret_cast<const u32x4_t*>(&As[(wm * 64 + i * 16 + (lane & 15)) * LD + (lane >> 4) * 8]);
+      bf[i] = *reinterpret_cast<const u32x4_t*>(&Bs[(wn * 64 + i * 16 + (lane & 15)) * LD + (lane >> 4) * 8]);
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) acc[i][j] = mfma_bf16(af[i], bf[j], acc[i][j]);
+    __syncthreads();
+  }
+  asm volatile("s_nop 15\n\ts_nop 7" ::: "memory");  // the matrix pipe's write-back before the results are read
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int n = n0 + wn * 64 + j * 16 + (lane & 15);
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int t = m0 + wm * 64 + i * 16 + (lane >> 4) * 4 + r;
+        if (t < a.T && n < a.N) lin_epilogue(a, g, t, n, acc[i][j][r], DIHIP_BF16);
+      }
+    }
+}
+
+// ------------------------------------------------------------------------------------------ weight-streaming kernel
+__device__ __forceinline__ float dot8_bf16(const u32x4_t& w, const u32x4_t& x, float acc) {
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    acc = __builtin_fmaf(__uint_as_float(w[i] << 16), __uint_as_float(x[i] << 16), acc);
+    acc = __builtin_fmaf(__uint_as_float(w[i] & 0xffff0000u), __uint_as_float(x[i] & 0xffff0000u), acc);
+  }
+  return acc;
+}
+
+// rows t0 .. t0 + tc (tc <= 4) of x staged as bf16 in LDS; wave w of block b owns weight rows (b * 4 + w) * 4 .. + 4.
+// K % 8 == 0 and 16-byte aligned weight rows (host-checked).
+template <int XT>
+__global__ __launch_bounds__(256) void linear_skinny_kernel(LinArgs a, int t0, int tc) {
+  extern __shared__ __attribute__((aligned(16))) uint16_t xsm[];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int g = blockIdx.y;
+  const size_t xoff = (size_t)(g % a.xgroups) * a.xg;
+  for (int idx = tid; idx < tc * a.K; idx += 256) {
+    const int t = idx / a.K, k = idx - t * a.K;
+    xsm[idx] = (uint16_t)f32_to_bf16_bits(load_ft<XT>(a.x, (size_t)(t0 + t) * a.ldx + xoff + k));
+  }
+  __syncthreads();
+  const int nb = (blockIdx.x * 4 + wave) * 4;
+  if (nb >= a.N) return;
+  const uint16_t* wp = (const uint16_t*)a.w + (size_t)g * a.N * a.K;
+  float acc[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int t = 0; t < 4; ++t) acc[i][t] = 0.f;
+  for (int k = lane * 8; k < a.K; k += 512) {
+    u32x4_t wv[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int n = min(nb + i, a.N - 1);
+      wv[i] = *reinterpret_cast<const u32x4_t*>(wp + (size_t)n * a.K + k);
+    }
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      if (t < tc) {
+        const u32x4_t xv = *reinterpret_cast<const u32x4_t*>(xsm + (size_t)t * a.K + k);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc[i][t] = dot8_bf16(wv[i], xv, acc[i][t]);
+      }
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      const float v = wave_sum(acc[i][t]);
+      if (lane == 0 && t < tc && nb + i < a.N) lin_epilogue(a, g, t0 + t, nb + i, v, DIHIP_BF16);
+    }
+}
+
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+}  // namespace
+}  // namespace dihip
+
+using namespace dihip;
+
+extern "C" int dihip_linear(void* stream, const void* x, int x_dtype, long ldx, long x_gstride, int x_groups, const void* w,
+                            int w_dtype, const void* bias, void* y, int y_dtype, long ldy, long y_gstride, const float* mul,
+                            long ldm, int T, int N, int K, int groups, int act, int act_lo, int act_hi, int math) {
+  DIHIP_REQUIRE(T >= 0 && N > 0 && K > 0 && groups > 0 && x_groups > 0, DIHIP_PARAM_ERROR, "linear: bad shape T %d N %d K %d groups %d", T, N, K, groups);
+  DIHIP_REQUIRE(seq_dtype_ok(x_dtype) && seq_dtype_ok(w_dtype) && seq_dtype_ok(y_dtype), DIHIP_PARAM_ERROR, "linear: f32 / bf16 only");
+  DIHIP_REQUIRE(x && w && y, DIHIP_PARAM_ERROR, "linear: null pointer");
+  DIHIP_REQUIRE(ldx >= K && ldy >= N && (!mul || ldm >= N), DIHIP_PARAM_ERROR, "linear: a row stride below the row length");
+  DIHIP_REQUIRE(math == DIHIP_MATH_F32 || math == DIHIP_MATH_BF16, DIHIP_PARAM_ERROR, "linear: unknown math mode %d", math);
+  DIHIP_REQUIRE(groups <= 65535, DIHIP_PARAM_ERROR, "linear: more than 65535 groups");
+  if (T == 0) return DIHIP_SUCCESS;
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  LinArgs a{x, ldx, x_gstride, x_groups, w, bias, y, ldy, y_gstride, mul, ldm, T, N, K, act, act_lo, act_hi, y_dtype, 0};
+  const size_t xe = x_dtype == DIHIP_F32 ? 4 : 2;
+  const bool vec = w_dtype == DIHIP_BF16 && K % 8 == 0 && aligned16(w) && aligned16(x) && (ldx * xe) % 16 == 0 &&
+                   (x_gstride * xe) % 16 == 0;
+  if (math == DIHIP_MATH_BF16 && w_dtype == DIHIP_BF16) {
+    static const bool no_skinny = env_off("DIHIP_LINEAR_SKINNY");
+    if (T <= 16 && vec && !no_skinny && (size_t)K * 2 * 4 <= 65536) {
+      for (int t0 = 0; t0 < T; t0 += 4) {
+        const int tc = T - t0 < 4 ? T - t0 : 4;
+        const dim3 grid((N + 15) / 16, groups);
+        if (x_dtype == DIHIP_F32) hipLaunchKernelGGL(linear_skinny_kernel<DIHIP_F32>, grid, dim3(256), (size_t)tc * K * 2, s, a, t0, tc);
+        else hipLaunchKernelGGL(linear_skinny_kernel<DIHIP_BF16>, grid, dim3(256), (size_t)tc * K * 2, s, a, t0, tc);
+      }
+      return launch_status();
+    }
+    const dim3 grid((N + 127) / 128, (T + 127) / 128, groups);
+    DIHIP_REQUIRE(grid.y <= 65535, DIHIP_PARAM_ERROR, "linear: too many rows for one launch");
+    if (x_dtype == DIHIP_F32) {
+      if (vec) hipLaunchKernelGGL((linear_mfma_kernel<DIHIP_F32, true>), grid, dim3(256), 0, s, a);
+      else hipLaunchKernelGGL((linear_mfma_kernel<DIHIP_F32, false>), grid, dim3(256), 0, s, a);
+    } else {
+      if (vec) hipLaunchKernelGGL((linear_mfma_kernel<DIHIP_BF16, true>), grid, dim3(256), 0, s, a);
+      else hipLaunchKernelGGL((linear_mfma_kernel<DIHIP_BF16, false>), grid, dim3(256), 0, s, a);
+    }
+    return launch_status();
+  }
+  a.round_ops = math == DIHIP_MATH_BF16;
+  const dim3 grid((N + 63) / 64, (T + 63) / 64, groups);
+  DIHIP_REQUIRE(grid.y <= 65535, DIHIP_PARAM_ERROR, "linear: too many rows for one launch");
+  if (x_dtype == DIHIP_F32 && w_dtype == DIHIP_F32) hipLaunchKernelGGL((linear_tile_kernel<DIHIP_F32, DIHIP_F32>), grid, dim3(256), 0, s, a);
+  else if (x_dtype == DIHIP_F32) hipLaunchKernelGGL((linear_tile_kernel<DIHIP_F32, DIHIP_BF16>), grid, dim3(256), 0, s, a);
+  else if (w_dtype == DIHIP_F32) hipLaunchKernelGGL((linear_tile_kernel<DIHIP_BF16, DIHIP_F32>), grid, dim3(256), 0, s, a);
+  else hipLaunchKernelGGL((linear_tile_kernel<DIHIP_BF16, DIHIP_BF16>), grid, dim3(256), 0, s, a);
+  return launch_status();
+}

@@ -1,0 +1,363 @@
+// seq_mixers.hip -- the token-mixing and residual-stream operators of the sequence engine (everything in f32):
+// embedding sums, strided RMS norms (also into the paged latent cache), the output-normed residual step with the
+// depth-weighted stream, windowed sink-softmax attention over shared latent rows, causal short convolutions and the
+// gated linear recurrence with per-slot state.
+#include <cstdarg>
+#include <cstdio>
+
+#include "seq_common.h"
+
+namespace dihip {
+namespace {
+
+// ------------------------------------------------------------------------------------------------ embedding
+__global__ __launch_bounds__(256) void embed_sum_kernel(float* __restrict__ h, const int32_t* __restrict__ ids, const void* __restrict__ table,
+                                                        const int32_t* __restrict__ rows2, const void* __restrict__ table2, int wdt, int K) {
+  const int t = blockIdx.x;
+  const size_t r1 = (size_t)ids[t] * K, r2 = table2 ? (size_t)rows2[t] * K : 0;
+  for (int k = threadIdx.x; k < K; k += 256) {
+    float v = ld_any(table, r1 + k, wdt);
+    if (table2) v += ld_any(table2, r2 + k, wdt);
+    h[(size_t)t * K + k] = v;
+  }
+}
+
+// ------------------------------------------------------------------------------------------------ norms
+// sum of squares of a row, k ascending per thread, one fixed tree over the block
+__device__ __forceinline__ float row_sumsq(const float* __restrict__ x, int K, float* red) {
+  float ss = 0.f;
+  for (int k = threadIdx.x; k < K; k += 256) {
+    const float v = x[k];
+    ss = __builtin_fmaf(v, v, ss);
+  }
+  return block256_sum(ss, red);
+}
+
+__global__ __launch_bounds__(256) void rmsnorm_strided_kernel(void* __restrict__ y, int ydt, long ldy, const float* __restrict__ x, long ldx,
+                                                              const int32_t* __restrict__ row_idx, const void* __restrict__ gamma, int wdt,
+                                                              float eps, int K) {
+  __shared__ float red[4];
+  const int i = blockIdx.x;
+  const float* xr = x + (size_t)(row_idx ? row_idx[i] : i) * ldx;
+  const float inv = 1.f / sqrtf(row_sumsq(xr, K, red) / (float)K + eps);
+  for (int k = threadIdx.x; k < K; k += 256) st_any(y, (size_t)i * ldy + k, ydt, xr[k] * inv * ld_any(gamma, k, wdt));
+}
+
+__global__ __launch_bounds__(256) void norm_span_append_kernel(void* const* __restrict__ spans, int span_stride, int span_len, int cdt,
+                                                               const float* __restrict__ x, long ldx, const void* __restrict__ gamma, int wdt,
+                                                               float eps, const int32_t* __restrict__ tok_slot,
+                                                               const int32_t* __restrict__ tok_pos, int K) {
+  __shared__ float red[4];
+  const int t = blockIdx.x;
+  const float* xr = x + (size_t)t * ldx;
+  const float inv = 1.f / sqrtf(row_sumsq(xr, K, red) / (float)K + eps);
+  const int pos = tok_pos[t];
+  void* span = spans[(size_t)tok_slot[t] * span_stride + pos / span_len];
+  const size_t base = (size_t)(pos % span_len) * K;
+  for (int k = threadIdx.x; k < K; k += 256) st_any(span, base + k, cdt, xr[k] * inv * ld_any(gamma, k, wdt));
+}
+
+__global__ __launch_bounds__(256) void norm_residual_mix_kernel(float* x_out, const float* x_in, const float* __restrict__ m,
+                                                                long ldm, const void* __restrict__ gamma, int wdt, float eps,
+                                                                float* __restrict__ stack, size_t stack_stride, const void* __restrict__ mix_w,
+                                                                int n_mix, float* __restrict__ x_mix, int K) {
+  __shared__ float red[4];
+  const int t = blockIdx.x;
+  const float* mr = m + (size_t)t * ldm;
+  const float inv = 1.f / sqrtf(row_sumsq(mr, K, red) / (float)K + eps);
+  const size_t row = (size_t)t * K;
+  for (int k = threadIdx.x; k < K; k += 256) {
+    const float xo = x_in[row + k] + mr[k] * inv * ld_any(gamma, k, wdt);
+    x_out[row + k] = xo;
+    if (n_mix > 0) {
+      stack[(size_t)(n_mix - 1) * stack_stride + row + k] = xo;
+      float mix = 0.f;
+      for (int j = 0; j + 1 < n_mix; ++j) mix = __builtin_fmaf(ld_any(mix_w, j, wdt), stack[(size_t)j * stack_stride + row + k], mix);
+      x_mix[row + k] = __builtin_fmaf(ld_any(mix_w, n_mix - 1, wdt), xo, mix);
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------------------------ latent attention
+// One workgroup per row, its 4 waves take the heads in turn.  A wave walks the row's window in chunks of 64 keys: lane j
+// scores key j (f32 dot over the R latent elements, r ascending), the chunk joins the running softmax (which starts at
+// the sink: maximum = sink, denominator = 1), then the lanes turn to the latent elements (lane l owns r = l, l + 64, ..)
+// and add the chunk's weighted rows.  Keys come from the cache only (the step's own rows were appended before).
+template <int CT, int RV>
+__global__ __launch_bounds__(256) void latent_attn_kernel(float* __restrict__ out, long ldo, const float* __restrict__ q, long ldq,
+                                                          void* const* __restrict__ spans, int span_stride, int span_len,
+                                                          const void* __restrict__ sink, int wdt, const int32_t* __restrict__ tok_slot,
+                                                          const int32_t* __restrict__ tok_pos, int H, int R, int window, float scale) {
+  __shared__ float qs[4][RV * 64];
+  __shared__ float ps[4][64];
+  const int t = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int pos = tok_pos[t];
+  const int j_lo = window > 0 ? max(0, pos - window + 1) : 0;
+  void* const* tab = spans + (size_t)tok_slot[t] * span_stride;
+  constexpr size_t ES = CT == DIHIP_F32 ? 4 : 2;
+  for (int h0 = 0; h0 < H; h0 += 4) {
+    const int h = h0 + wave;
+    const bool live = h < H;
+    __syncthreads();  // qs / ps of the head before are no longer read
+    if (live)
+      for (int r = lane; r < R; r += 64) qs[wave][r] = q[(size_t)t * ldq + (size_t)h * R + r];
+    __syncthreads();
+    float mx = -INFINITY, den = 0.f;
+    if (sink) { mx = ld_any(sink, h < H ? h : 0, wdt); den = 1.f; }
+    float acc[RV];
+#pragma unroll
+    for (int v = 0; v < RV; ++v) acc[v] = 0.f;
+    for (int j0 = j_lo; j0 <= pos; j0 += 64) {  // the same trip count in every wave of the block
+      const int j = j0 + lane;
+      const bool valid = live && j <= pos;
+      float s = -INFINITY;
+      if (valid) {
+        const char* row = (const char*)tab[j / span_len] + (size_t)(j % span_len) * R * ES;
+        float d = 0.f;
+        for (int r = 0; r < R; ++r) d = __builtin_fmaf(qs[wave][r], load_ft<CT>(row, r), d);
+        s = d * scale;
+      }
+      const float mnew = fmaxf(mx, wave_max(s));
+      const float corr = mx == -INFINITY ? 0.f : expf(mx - mnew);
+      const float p = valid ? expf(s - mnew) : 0.f;
+      den = den * corr + wave_sum(p);
+#pragma unroll
+      for (int v = 0; v < RV; ++v) acc[v] *= corr;
+      mx = mnew;
+      ps[wave][lane] = p;
+      __syncthreads();
+      if (live) {
+        const int cnt = min(64, pos - j0 + 1);
+        for (int jj = 0; jj < cnt; ++jj) {
+          const int jk = j0 + jj;
+          const char* row = (const char*)tab[jk / span_len] + (size_t)(jk % span_len) * R * ES;
+          const float pj = ps[wave][jj];
+#pragma unroll
+          for (int v = 0; v < RV; ++v) {
+            const int r = v * 64 + lane;
+            if (r < R) acc[v] = __builtin_fmaf(pj, load_ft<CT>(row, r), acc[v]);
+          }
+        }
+      }
+      __syncthreads();
+    }
+    if (live) {
+#pragma unroll
+      for (int v = 0; v < RV; ++v) {
+        const int r = v * 64 + lane;
+        if (r < R) out[(size_t)t * ldo + (size_t)h * R + r] = acc[v] / den;
+      }
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------------------------ short convolution
+__global__ __launch_bounds__(256) void causal_conv_state_kernel(float* __restrict__ u, long ldu, const float* __restrict__ x, long ldx,
+                                                                const void* __restrict__ w, const void* __restrict__ bias, int wdt,
+                                                                const float* __restrict__ tail, const int32_t* __restrict__ tok_slot,
+                                                                const int32_t* __restrict__ tok_off, int C, int taps) {
+  const int t = blockIdx.x, c = blockIdx.y * 256 + threadIdx.x;
+  if (c >= C) return;
+  const int off = tok_off[t], nt = taps - 1;
+  const float* tl = tail + (size_t)tok_slot[t] * nt * C;
+  float acc = 0.f;
+  for (int k = 0; k < taps; ++k) {
+    const int d = nt - k, o = off - d;
+    const float v = o >= 0 ? x[(size_t)(t - d) * ldx + c] : tl[(size_t)(nt + o) * C + c];
+    acc = __builtin_fmaf(ld_any(w, (size_t)c * taps + k, wdt), v, acc);
+  }
+  if (bias) acc += ld_any(bias, c, wdt);
+  u[(size_t)t * ldu + c] = acc;
+}
+
+__global__ __launch_bounds__(256) void conv_tail_update_kernel(float* __restrict__ tail, const float* __restrict__ x, long ldx,
+                                                               const int32_t* __restrict__ ent_slot, const int32_t* __restrict__ ent_row0,
+                                                               const int32_t* __restrict__ ent_count, int C, int taps) {
+  const int e = blockIdx.x, c = blockIdx.y * 256 + threadIdx.x;
+  if (c >= C) return;
+  const int nt = taps - 1, cnt = ent_count[e], row0 = ent_row0[e];
+  float* tl = tail + (size_t)ent_slot[e] * nt * C;
+  float old[16];
+#pragma unroll
+  for (int i = 0; i < 16; ++i) old[i] = i < nt ? tl[(size_t)i * C + c] : 0.f;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    if (i < nt) {
+      const int o = cnt - nt + i;  // index inside the portion of the input that becomes tail row i
+      float v;
+      if (o >= 0) v = x[(size_t)(row0 + o) * ldx + c];
+      else {
+        v = 0.f;
+#pragma unroll
+        for (int j = 0; j < 16; ++j)
+          if (j == nt + o) v = old[j];
+      }
+      tl[(size_t)i * C + c] = v;
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------------------------ gated recurrence
+__device__ __forceinline__ float softplus_f32(float x) { return x > 20.f ? x : log1pf(expf(x)); }
+
+__global__ __launch_bounds__(64) void gated_recurrence_kernel(float* __restrict__ out, long ldo, const float* __restrict__ r, const float* __restrict__ ig,
+                                                              long ldg, const float* __restrict__ u, long ldu, const float* __restrict__ y, long ldy,
+                                                              const void* __restrict__ lam, int wdt, float decay, float* __restrict__ state,
+                                                              const int32_t* __restrict__ ent_slot, const int32_t* __restrict__ ent_row0,
+                                                              const int32_t* __restrict__ ent_count, int C) {
+  const int e = blockIdx.x, c = blockIdx.y * 64 + threadIdx.x;
+  if (c >= C) return;
+  const int cnt = ent_count[e], row0 = ent_row0[e];
+  float* sp = state + (size_t)ent_slot[e] * C + c;
+  float S = *sp;
+  const float k = -decay * softplus_f32(ld_any(lam, c, wdt));
+  constexpr int U = 8;
+  for (int i0 = 0; i0 < cnt; i0 += U) {
+    float rv[U], iv[U], uv[U], yv[U];
+#pragma unroll
+    for (int j = 0; j < U; ++j) {
+      const size_t t = (size_t)(row0 + min(i0 + j, cnt - 1));
+      rv[j] = r[t * ldg + c]; iv[j] = ig[t * ldg + c]; uv[j] = u[t * ldu + c]; yv[j] = y[t * ldy + c];
+    }
+#pragma unroll
+    for (int j = 0; j < U; ++j) {
+      if (i0 + j < cnt) {
+        const float la = k * rv[j];
+        const float a = expf(la);
+        const float g = sqrtf(-expm1f(2.f * la)) * iv[j] * uv[j];
+        S = __builtin_fmaf(a, S, g);
+        out[(size_t)(row0 + i0 + j) * ldo + c] = S * yv[j];
+      }
+    }
+  }
+  *sp = S;
+}
+
+static thread_local char g_seq_error[512] = "";
+
+}  // namespace
+
+void set_last_error(const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_seq_error, sizeof(g_seq_error), fmt, ap);
+  va_end(ap);
+}
+int env_int(const char* name, int dflt) {
+  const char* e = getenv(name);
+  return e ? atoi(e) : dflt;
+}
+bool env_off(const char* name) {
+  const char* e = getenv(name);
+  return e && e[0] == '0';
+}
+
+}  // namespace dihip
+
+using namespace dihip;
+
+extern "C" {
+
+const char* dihip_seq_version(void) { return "dashinfer-hip-seq 0.1.0 (gfx950)"; }
+const char* dihip_seq_last_error(void) { return g_seq_error; }
+
+int dihip_embed_sum(void* stream, float* h, const int32_t* ids, const void* table, const int32_t* rows2, const void* table2,
+                    int w_dtype, int T, int K) {
+  DIHIP_REQUIRE(T >= 0 && K > 0 && h && ids && table && (!table2 || rows2) && seq_dtype_ok(w_dtype), DIHIP_PARAM_ERROR, "embed_sum: bad argument");
+  if (T == 0) return DIHIP_SUCCESS;
+  hipLaunchKernelGGL(embed_sum_kernel, dim3(T), dim3(256), 0, reinterpret_cast<hipStream_t>(stream), h, ids, table, rows2, table2, w_dtype, K);
+  return launch_status();
+}
+
+int dihip_rmsnorm_strided(void* stream, void* y, int y_dtype, long ldy, const float* x, long ldx, const int32_t* row_idx,
+                          const void* gamma, int w_dtype, float eps, int M, int K) {
+  DIHIP_REQUIRE(M >= 0 && K > 0 && y && x && gamma && ldy >= K && ldx >= K && seq_dtype_ok(y_dtype) && seq_dtype_ok(w_dtype),
+                DIHIP_PARAM_ERROR, "rmsnorm_strided: bad argument");
+  if (M == 0) return DIHIP_SUCCESS;
+  hipLaunchKernelGGL(rmsnorm_strided_kernel, dim3(M), dim3(256), 0, reinterpret_cast<hipStream_t>(stream), y, y_dtype, ldy, x, ldx, row_idx,
+                     gamma, w_dtype, eps, K);
+  return launch_status();
+}
+
+int dihip_norm_span_append(void* stream, void* const* spans, int span_stride, int span_len, int cache_dtype, const float* x, long ldx,
+                           const void* gamma, int w_dtype, float eps, const int32_t* tok_slot, const int32_t* tok_pos, int T, int K) {
+  DIHIP_REQUIRE(T >= 0 && K > 0 && spans && x && gamma && tok_slot && tok_pos && span_stride > 0 && span_len > 0 && ldx >= K &&
+                    seq_dtype_ok(cache_dtype) && seq_dtype_ok(w_dtype), DIHIP_PARAM_ERROR, "norm_span_append: bad argument");
+  if (T == 0) return DIHIP_SUCCESS;
+  hipLaunchKernelGGL(norm_span_append_kernel, dim3(T), dim3(256), 0, reinterpret_cast<hipStream_t>(stream), spans, span_stride, span_len,
+                     cache_dtype, x, ldx, gamma, w_dtype, eps, tok_slot, tok_pos, K);
+  return launch_status();
+}
+
+int dihip_norm_residual_mix(void* stream, float* x_out, const float* x_in, const float* m, long ldm, const void* gamma, int w_dtype,
+                            float eps, float* stack, size_t stack_stride, const void* mix_w, int n_mix, float* x_mix, int T, int K) {
+  DIHIP_REQUIRE(T >= 0 && K > 0 && x_out && x_in && m && gamma && ldm >= K && seq_dtype_ok(w_dtype), DIHIP_PARAM_ERROR,
+                "norm_residual_mix: bad argument");
+  DIHIP_REQUIRE(n_mix == 0 || (stack && mix_w && x_mix && stack_stride >= (size_t)T * K && x_mix != x_out), DIHIP_PARAM_ERROR,
+                "norm_residual_mix: the depth mix needs the stack, its weights and an output of its own");
+  if (T == 0) return DIHIP_SUCCESS;
+  hipLaunchKernelGGL(norm_residual_mix_kernel, dim3(T), dim3(256), 0, reinterpret_cast<hipStream_t>(stream), x_out, x_in, m, ldm, gamma,
+                     w_dtype, eps, stack, stack_stride, mix_w, n_mix, x_mix, K);
+  return launch_status();
+}
+
+int dihip_latent_window_attn(void* stream, float* out, long ldo, const float* q, long ldq, void* const* spans, int span_stride,
+                             int span_len, int cache_dtype, const void* sink, int w_dtype, const int32_t* tok_slot,
+                             const int32_t* tok_pos, int T, int H, int R, int window, float scale, int math) {
+  DIHIP_REQUIRE(T >= 0 && H > 0 && R > 0 && out && q && spans && tok_slot && tok_pos && span_stride > 0 && span_len > 0 &&
+                    ldo >= (long)H * R && ldq >= (long)H * R && seq_dtype_ok(cache_dtype) && seq_dtype_ok(w_dtype),
+                DIHIP_PARAM_ERROR, "latent_window_attn: bad argument");
+  DIHIP_REQUIRE(R <= 1024, DIHIP_EXCEED_LIMIT_ERROR, "latent_window_attn: latent rows of more than 1024 elements (%d)", R);
+  (void)math;
+  if (T == 0) return DIHIP_SUCCESS;
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  auto go = [&](auto ct, auto rv) {
+    constexpr int CT = decltype(ct)::value, RV = decltype(rv)::value;
+    hipLaunchKernelGGL((latent_attn_kernel<CT, RV>), dim3(T), dim3(256), 0, s, out, ldo, q, ldq, spans, span_stride, span_len, sink,
+                       w_dtype, tok_slot, tok_pos, H, R, window, scale);
+  };
+  auto by_r = [&](auto ct) {
+    if (R <= 64) go(ct, std::integral_constant<int, 1>{});
+    else if (R <= 128) go(ct, std::integral_constant<int, 2>{});
+    else if (R <= 256) go(ct, std::integral_constant<int, 4>{});
+    else if (R <= 512) go(ct, std::integral_constant<int, 8>{});
+    else go(ct, std::integral_constant<int, 16>{});
+  };
+  if (cache_dtype == DIHIP_F32) by_r(std::integral_constant<int, DIHIP_F32>{});
+  else by_r(std::integral_constant<int, DIHIP_BF16>{});
+  return launch_status();
+}
+
+int dihip_causal_conv_state(void* stream, float* u, long ldu, const float* x, long ldx, const void* w, const void* bias, int w_dtype,
+                            const float* tail, const int32_t* tok_slot, const int32_t* tok_off, int T, int C, int taps) {
+  DIHIP_REQUIRE(T >= 0 && C > 0 && taps >= 1 && taps <= 16 && u && x && w && (tail || taps == 1) && tok_slot && tok_off && ldu >= C &&
+                    ldx >= C && seq_dtype_ok(w_dtype), DIHIP_PARAM_ERROR, "causal_conv_state: bad argument (1 <= taps <= 16)");
+  if (T == 0) return DIHIP_SUCCESS;
+  hipLaunchKernelGGL(causal_conv_state_kernel, dim3(T, (C + 255) / 256), dim3(256), 0, reinterpret_cast<hipStream_t>(stream), u, ldu, x, ldx,
+                     w, bias, w_dtype, tail, tok_slot, tok_off, C, taps);
+  return launch_status();
+}
+
+int dihip_conv_tail_update(void* stream, float* tail, const float* x, long ldx, const int32_t* ent_slot, const int32_t* ent_row0,
+                           const int32_t* ent_count, int E, int C, int taps) {
+  DIHIP_REQUIRE(E >= 0 && C > 0 && taps >= 1 && taps <= 16 && x && ent_slot && ent_row0 && ent_count && ldx >= C, DIHIP_PARAM_ERROR,
+                "conv_tail_update: bad argument (1 <= taps <= 16)");
+  if (E == 0 || taps == 1) return DIHIP_SUCCESS;
+  DIHIP_REQUIRE(tail, DIHIP_PARAM_ERROR, "conv_tail_update: null state");
+  hipLaunchKernelGGL(conv_tail_update_kernel, dim3(E, (C + 255) / 256), dim3(256), 0, reinterpret_cast<hipStream_t>(stream), tail, x, ldx,
+                     ent_slot, ent_row0, ent_count, C, taps);
+  return launch_status();
+}
+
+int dihip_gated_recurrence(void* stream, float* out, long ldo, const float* r, const float* i, long ldg, const float* u, long ldu,
+                           const float* y, long ldy, const void* lam, int w_dtype, float decay, float* state, const int32_t* ent_slot,
+                           const int32_t* ent_row0, const int32_t* ent_count, int E, int C) {
+  DIHIP_REQUIRE(E >= 0 && C > 0 && out && r && i && u && y && lam && state && ent_slot && ent_row0 && ent_count && ldo >= C &&
+                    ldg >= C && ldu >= C && ldy >= C && seq_dtype_ok(w_dtype), DIHIP_PARAM_ERROR, "gated_recurrence: bad argument");
+  if (E == 0) return DIHIP_SUCCESS;
+  hipLaunchKernelGGL(gated_recurrence_kernel, dim3(E, (C + 63) / 64), dim3(64), 0, reinterpret_cast<hipStream_t>(stream), out, ldo, r, i, ldg,
+                     u, ldu, y, ldy, lam, w_dtype, decay, state, ent_slot, ent_row0, ent_count, C);
+  return launch_status();
+}
+
+}  // extern "C"

@@ -352,8 +352,9 @@ class SpanPool:
     reference's span-attention test (test_quant_none.cpp:479-506).  Stands in for the
     reference's CacheFrameManager / CacheSpanManager (out of scope, host code)."""
 
-    def __init__(self, num_spans, g, S, H, mode, dtype, device="cuda", stride=7):
-        self.nbytes = span_bytes(g, S, H, mode, dtype)
+    def __init__(self, num_spans, g, S, H, mode, dtype, device="cuda", stride=7, nbytes=None):
+        # nbytes: the span size when the caller knows it (16- and 32-bit spans of mode "none" are g * S * H elements)
+        self.nbytes = int(nbytes) if nbytes is not None else span_bytes(g, S, H, mode, dtype)
         self.aligned = (self.nbytes + 255) // 256 * 256
         self.pool = torch.zeros(num_spans * self.aligned, dtype=torch.uint8, device=device)
         self.g, self.S, self.H, self.mode, self.dtype = g, S, H, mode, dtype
@@ -366,6 +367,14 @@ class SpanPool:
     def alloc(self):
         idx = self.free.pop(0)
         return self.pool.data_ptr() + idx * self.aligned, idx
+
+    def release(self, idx):
+        """Give span idx back; it is handed out again after the spans that are free now."""
+        assert 0 <= idx and idx not in self.free
+        self.free.append(idx)
+
+    def span_ptr(self, idx):
+        return self.pool.data_ptr() + idx * self.aligned
 
     def span_view(self, idx):
         return self.pool[idx * self.aligned: idx * self.aligned + self.nbytes]

@@ -1,0 +1,91 @@
+/* dashinfer_hip_seq.h -- C-ABI of libdashinfer_hip_seq.so: the operators of the ragged-batch sequence engine
+ * (dash-infer_amd/engine.py): row-major linear layers, strided norms, the depth-weighted residual stream, windowed
+ * attention over a paged latent cache with a softmax sink, causal short convolutions and gated linear recurrences with
+ * per-sequence state slots.  Conventions are those of dashinfer_hip.h: plain pointers and sizes, `stream` = hipStream_t,
+ * status 0 = success, dihip_seq_last_error() holds the text of the last failure of the calling thread; dtype codes
+ * DIHIP_F32 / DIHIP_BF16.
+ *
+ * A step's tokens are ONE flat list of T rows (portions of prompts beside single decoded tokens).  Per row:
+ *   tok_slot[t]  the state slot of the row's sequence,   tok_pos[t]  its position in the sequence (from 0),
+ *   tok_off[t]   its index inside the portion this step brings (0 = the portion's first row).
+ * Paged caches are tables of span pointers, one row of `span_stride` pointers per slot (as dihip_kv_append takes them);
+ * a span holds `span_len` consecutive positions.  Nothing here depends on what else is in the batch: every output row
+ * is computed by the same instructions in the same order whatever T is. */
+#ifndef DASHINFER_HIP_SEQ_H_
+#define DASHINFER_HIP_SEQ_H_
+#include <stddef.h>
+#include <stdint.h>
+
+#include "dashinfer_hip.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+const char* dihip_seq_version(void);
+const char* dihip_seq_last_error(void);
+
+/* math of dihip_linear: EXACT = every product and sum in f32, k ascending; BF16 = operands rounded to bf16, f32
+ * accumulation on the matrix cores (T > DIHIP_LINEAR_SKINNY_ROWS) or in a weight-streaming dot-product kernel */
+enum { DIHIP_MATH_F32 = 0, DIHIP_MATH_BF16 = 1 };
+
+/* y[g][t, n] = epilogue( sum_k x[g % x_groups][t, k] * w[g][n, k] + bias[g][n] ),  g < groups, t < T, n < N
+ *   x: [T, .] rows of stride ldx, group g starts at column (g % x_groups) * x_gstride;  w: [groups][N][K] row-major,
+ *   bias: [groups][N] or NULL (w_dtype);  y: rows of stride ldy, group g at column g * y_gstride;
+ *   epilogue: activation `act` on the columns act_lo <= g * N + n < act_hi, then * mul[t, g * y_gstride + n] (rows of
+ *   stride ldm, f32; NULL: none). */
+int dihip_linear(void* stream, const void* x, int x_dtype, long ldx, long x_gstride, int x_groups,
+                 const void* w, int w_dtype, const void* bias, void* y, int y_dtype, long ldy, long y_gstride,
+                 const float* mul, long ldm, int T, int N, int K, int groups, int act, int act_lo, int act_hi, int math);
+
+/* h[t, :] = float(table[ids[t], :]) + float(table2[rows2[t], :])   (table2 NULL: the first term alone) */
+int dihip_embed_sum(void* stream, float* h, const int32_t* ids, const void* table, const int32_t* rows2,
+                    const void* table2, int w_dtype, int T, int K);
+
+/* y[i, :] = x[r, :] / sqrt(mean(x[r, :]^2) + eps) * gamma,  r = row_idx ? row_idx[i] : i;  x f32 rows of stride ldx */
+int dihip_rmsnorm_strided(void* stream, void* y, int y_dtype, long ldy, const float* x, long ldx,
+                          const int32_t* row_idx, const void* gamma, int w_dtype, float eps, int M, int K);
+/* the same norm, written into the paged cache at (tok_slot[t], tok_pos[t]): span row of K elements of cache_dtype */
+int dihip_norm_span_append(void* stream, void* const* spans, int span_stride, int span_len, int cache_dtype,
+                           const float* x, long ldx, const void* gamma, int w_dtype, float eps,
+                           const int32_t* tok_slot, const int32_t* tok_pos, int T, int K);
+
+/* The residual step with the norm on the sublayer's OUTPUT and the depth-weighted stream:
+ *   x_out[t] = x_in[t] + rmsnorm(m[t]; gamma, eps)
+ *   n_mix > 0:  stack[n_mix - 1][t] = x_out[t];  x_mix[t] = sum_{j < n_mix} mix_w[j] * stack[j][t]
+ * stack: [.][stack_stride] f32 (stack_stride >= T * K elements per level); x_out may alias x_in. */
+int dihip_norm_residual_mix(void* stream, float* x_out, const float* x_in, const float* m, long ldm,
+                            const void* gamma, int w_dtype, float eps, float* stack, size_t stack_stride,
+                            const void* mix_w, int n_mix, float* x_mix, int T, int K);
+
+/* Windowed attention of every row over its sequence's cached latent rows, all heads sharing the cache:
+ *   s_j = scale * q[t, h, :] . c_j   for  0 <= tok_pos[t] - j < window  (window <= 0: every j <= tok_pos[t]),
+ *   p = softmax over {s_j} and one extra logit sink[h] that has no value (sink NULL: none),
+ *   out[t, h, :] = sum_j p_j c_j.
+ * q, out: f32 [T, H, R] (rows of stride ldq / ldo); the cache holds rows of R elements of cache_dtype. */
+int dihip_latent_window_attn(void* stream, float* out, long ldo, const float* q, long ldq, void* const* spans,
+                             int span_stride, int span_len, int cache_dtype, const void* sink, int w_dtype,
+                             const int32_t* tok_slot, const int32_t* tok_pos, int T, int H, int R, int window,
+                             float scale, int math);
+
+/* u[t, c] = bias[c] + sum_{k < taps} w[c, k] * src(t, k),  src = x[t - (taps - 1 - k), c] inside the portion, else the
+ * slot's tail state [slots][taps - 1][C] f32 (the last taps - 1 inputs of the sequence; zeros at its start) */
+int dihip_causal_conv_state(void* stream, float* u, long ldu, const float* x, long ldx, const void* w,
+                            const void* bias, int w_dtype, const float* tail, const int32_t* tok_slot,
+                            const int32_t* tok_off, int T, int C, int taps);
+/* after it: tail <- the last taps - 1 inputs of every portion (ent_slot / ent_row0 / ent_count: [E]) */
+int dihip_conv_tail_update(void* stream, float* tail, const float* x, long ldx, const int32_t* ent_slot,
+                           const int32_t* ent_row0, const int32_t* ent_count, int E, int C, int taps);
+
+/* Real-gated linear recurrence, per channel c and portion, rows in order:
+ *   a = exp(-decay * r[t, c] * softplus(lam[c]));  S = a * S + sqrt(1 - a^2) * i[t, c] * u[t, c];  out[t, c] = S * y[t, c]
+ * S: state [slots][C] f32, read at the portion's start and written back at its end.  r, i, u, y, out: f32 rows. */
+int dihip_gated_recurrence(void* stream, float* out, long ldo, const float* r, const float* i, long ldg,
+                           const float* u, long ldu, const float* y, long ldy, const void* lam, int w_dtype,
+                           float decay, float* state, const int32_t* ent_slot, const int32_t* ent_row0,
+                           const int32_t* ent_count, int E, int C);
+
+#ifdef __cplusplus
+}
+#endif
+#endif
