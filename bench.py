@@ -1031,7 +1031,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=64)
     ap.add_argument("--warmup", type=int, default=8)
-    ap.add_argument("--workload", default="int4_b1", choices=list(WORKLOADS) + ["launch_selftest"])  # int4_b1 = the headline configuration
+    ap.add_argument("--workload", default="int4_b1", choices=list(WORKLOADS) + ["launch_selftest", "modanex_layers"])  # int4_b1 = the headline configuration
     ap.add_argument("--layers", type=int, default=None, help="debug: fewer decoder layers (result marked invalid)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-graph", action="store_true", help="debug: eager launches instead of hipGraph replay")
@@ -1085,6 +1085,16 @@ def main():
         comm = decoder.make_comm(rank, world, torch.device("cuda", local_rank), backend=os.environ.get("DIHIP_TP_ALLREDUCE", "auto"),
                                  allow_labelled_fallback=True)
 
+    if args.workload == "modanex_layers":
+        # the sequence engine on random Modanex models of real layer sizes, beside Qwen2 layers of equal size (dash-infer_amd/seq_bench.py)
+        assert world == 1, "modanex_layers is a one-GPU workload"
+        from dash_infer_amd import seq_bench
+        out = seq_bench.run(args)
+        os.makedirs(os.path.join(ROOT, "gpurun_out"), exist_ok=True)
+        with open(os.path.join(ROOT, "gpurun_out", "bench_modanex_layers.json"), "w") as f:
+            json.dump(out, f, indent=1)
+        print(json.dumps(out), flush=True)
+        return
     wbits, group, kv_mode, batch, gptq = WORKLOADS[args.workload]
     if args.workload == "prefill_2048":
         assert world == 1, "prefill_2048 is a one-GPU workload"

@@ -246,9 +246,10 @@ extern "C" int dihip_linear(void* stream, const void* x, int x_dtype, long ldx, 
                    (x_gstride * xe) % 16 == 0;
   if (math == DIHIP_MATH_BF16 && w_dtype == DIHIP_BF16) {
     static const bool no_skinny = env_off("DIHIP_LINEAR_SKINNY");
-    if (T <= 16 && vec && !no_skinny && (size_t)K * 2 * 4 <= 65536) {
-      for (int t0 = 0; t0 < T; t0 += 4) {
-        const int tc = T - t0 < 4 ? T - t0 : 4;
+    const int tmax = K <= 8192 ? 4 : (K <= 16384 ? 2 : 1);  // rows whose bf16 copy fits 64 KB of LDS
+    if (T <= 4 * tmax && vec && !no_skinny && K <= 32768) {
+      for (int t0 = 0; t0 < T; t0 += tmax) {
+        const int tc = T - t0 < tmax ? T - t0 : tmax;
         const dim3 grid((N + 15) / 16, groups);
         if (x_dtype == DIHIP_F32) hipLaunchKernelGGL(linear_skinny_kernel<DIHIP_F32>, grid, dim3(256), (size_t)tc * K * 2, s, a, t0, tc);
         else hipLaunchKernelGGL(linear_skinny_kernel<DIHIP_BF16>, grid, dim3(256), (size_t)tc * K * 2, s, a, t0, tc);

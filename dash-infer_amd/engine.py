@@ -93,6 +93,7 @@ class SeqEngine:
             o += n
         ctx = StepContext(T, E, *parts, math=model.math, eps=model.eps)
         ctx.taps = taps
+        ctx.max_count, ctx.max_pos = max(ecnt), max(tpos)
         x = model.forward(ctx)
         if not want:
             return None

@@ -23,6 +23,7 @@ class StepContext:
         self.ids, self.rows2, self.tok_slot, self.tok_pos, self.tok_off = ids, rows2, tok_slot, tok_pos, tok_off
         self.ent_slot, self.ent_row0, self.ent_count, self.want_rows = ent_slot, ent_row0, ent_count, want_rows
         self.math, self.eps = math, eps
+        self.max_count, self.max_pos = T, 0     # host numbers: the largest portion and the last position of the step
         self.taps = None    # layer index -> [T, .] intermediate (diagnostics; None: off)
 
 
@@ -49,6 +50,7 @@ class LatentWindowAttention:
         else:
             self.table = state.tables[kv_from_key]
             assert self.table.row_elems == kv_rank, "a shared latent cache must have this layer's rank"
+        self.mc = so.latent_attn_mc_supported(self.table) and (heads * kv_rank) % 4 == 0
 
     def __call__(self, ctx, h):
         a = so.linear(h, self.w_in, act="sigmoid", act_cols=(self.g_lo, self.n_in), math=ctx.math)
@@ -57,7 +59,11 @@ class LatentWindowAttention:
         if self.owns_cache:
             so.norm_span_append(self.table, a[:, self.c_lo: self.g_lo], self.dkv_norm, ctx.eps, ctx.tok_slot, ctx.tok_pos)
         ql = so.linear(q, self.uk_t, groups=self.H, math=ctx.math)
-        ol = so.latent_window_attn(ql, self.table, self.sink, ctx.tok_slot, ctx.tok_pos, self.H, self.window, self.scale, math=ctx.math)
+        if ctx.math == so.MATH_BF16 and self.mc:
+            ol = so.latent_window_attn_mc(ql, self.table, self.sink, ctx.tok_pos, ctx.ent_slot, ctx.ent_row0, ctx.ent_count, ctx.max_count,
+                                          ctx.max_pos, self.H, self.window, self.scale)
+        else:
+            ol = so.latent_window_attn(ql, self.table, self.sink, ctx.tok_slot, ctx.tok_pos, self.H, self.window, self.scale, math=ctx.math)
         og = so.linear(ol, self.uv, groups=self.H, mul=a[:, self.g_lo:], math=ctx.math)
         return so.linear(og, self.o, math=ctx.math)
 

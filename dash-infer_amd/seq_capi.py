@@ -26,6 +26,10 @@ _SIGS = {
     "dihip_norm_span_append": (i32, [vp, vp, i32, i32, i32, vp, lng, vp, i32, f32, vp, vp, i32, i32]),
     "dihip_norm_residual_mix": (i32, [vp, vp, vp, vp, lng, vp, i32, f32, vp, sz, vp, i32, vp, i32, i32]),
     "dihip_latent_window_attn": (i32, [vp, vp, lng, vp, lng, vp, i32, i32, i32, vp, i32, vp, vp, i32, i32, i32, i32, f32, i32]),
+    "dihip_latent_window_attn_mc_supported": (i32, [i32, i32, i32]),
+    "dihip_latent_window_attn_mc_workspace_bytes": (sz, [i32, i32, i32, i32]),
+    "dihip_latent_window_attn_mc": (i32, [vp, vp, lng, vp, lng, vp, i32, i32, vp, i32, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, f32, i32,
+                                          vp, sz]),
     "dihip_causal_conv_state": (i32, [vp, vp, lng, vp, lng, vp, vp, i32, vp, vp, vp, i32, i32, i32]),
     "dihip_conv_tail_update": (i32, [vp, vp, vp, lng, vp, vp, vp, i32, i32, i32]),
     "dihip_gated_recurrence": (i32, [vp, vp, lng, vp, vp, lng, vp, lng, vp, lng, vp, i32, f32, vp, vp, vp, vp, i32, i32]),

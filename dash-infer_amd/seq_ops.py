@@ -101,6 +101,29 @@ def latent_window_attn(q, table, sink, tok_slot, tok_pos, H, window, scale, math
     return o
 
 
+def latent_attn_mc_supported(table):
+    return bool(lib().dihip_latent_window_attn_mc_supported(table.row_elems, table.span_len, _DT[table.dtype]))
+
+
+def latent_window_attn_mc(q, table, sink, tok_pos, ent_slot, ent_row0, ent_count, max_count, max_pos, H, window, scale, out=None, nsplit=None):
+    """the matrix-core form (bf16 cache): rows as portions; max_count / max_pos: the largest portion and position of the step
+    (host numbers: they size the grid and the split of the key walk)"""
+    T, R, E = q.shape[0], table.row_elems, ent_slot.shape[0]
+    o = out if out is not None else torch.empty(T, H * R, dtype=torch.float32, device=q.device)
+    if nsplit is None:       # fill the chip: ~2 workgroups per CU; at least 4 key tiles (128 keys) per workgroup
+        blocks = max(1, E * ((max_count * H + 63) // 64))
+        keys = min(max_pos + 1, window) if window > 0 else max_pos + 1
+        nsplit = max(1, min(512 // blocks, (keys + 127) // 128))
+    ws = None
+    if nsplit > 1:
+        ws = torch.empty(int(lib().dihip_latent_window_attn_mc_workspace_bytes(T, H, R, nsplit)), dtype=torch.uint8, device=q.device)
+    check(lib().dihip_latent_window_attn_mc(stream(), ptr(o), _rows(o), ptr(q), _rows(q), ptr(table.ptrs), table.max_spans, table.span_len,
+                                            ptr(sink), dt(sink) if sink is not None else 0, ptr(tok_pos), ptr(ent_slot), ptr(ent_row0),
+                                            ptr(ent_count), E, int(max_count), T, H, R, int(window), float(scale), int(nsplit), ptr(ws),
+                                            ws.numel() if ws is not None else 0), "dihip_latent_window_attn_mc")
+    return o
+
+
 def causal_conv_state(x, w, bias, tail, tok_slot, tok_off, out=None):
     T, Cn = x.shape
     taps = w.shape[1]

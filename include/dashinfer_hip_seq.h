@@ -68,6 +68,19 @@ int dihip_latent_window_attn(void* stream, float* out, long ldo, const float* q,
                              const int32_t* tok_slot, const int32_t* tok_pos, int T, int H, int R, int window,
                              float scale, int math);
 
+/* The same attention on the matrix cores for a bf16 cache (R a multiple of 32 up to 512, span_len a multiple of 32; see
+ * .._supported): the rows are given as portions (ent_*: [E], rows ent_row0 .. + ent_count of one slot at consecutive
+ * positions from tok_pos[ent_row0]; max_count = the largest ent_count).  nsplit > 1 splits every row's key walk over
+ * that many workgroups (few rows: decoding) and merges the partial softmax records in a second launch through `ws`
+ * (.._workspace_bytes).  Operands are rounded to bf16, sums are f32; a row's result depends on the tiling only by rounding. */
+int dihip_latent_window_attn_mc_supported(int R, int span_len, int cache_dtype);
+size_t dihip_latent_window_attn_mc_workspace_bytes(int T, int H, int R, int nsplit);
+int dihip_latent_window_attn_mc(void* stream, float* out, long ldo, const float* q, long ldq, void* const* spans,
+                                int span_stride, int span_len, const void* sink, int w_dtype, const int32_t* tok_pos,
+                                const int32_t* ent_slot, const int32_t* ent_row0, const int32_t* ent_count, int E,
+                                int max_count, int T, int H, int R, int window, float scale, int nsplit, void* ws,
+                                size_t ws_bytes);
+
 /* u[t, c] = bias[c] + sum_{k < taps} w[c, k] * src(t, k),  src = x[t - (taps - 1 - k), c] inside the portion, else the
  * slot's tail state [slots][taps - 1][C] f32 (the last taps - 1 inputs of the sequence; zeros at its start) */
 int dihip_causal_conv_state(void* stream, float* u, long ldu, const float* x, long ldx, const void* w,

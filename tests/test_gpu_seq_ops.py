@@ -250,3 +250,39 @@ def test_gated_recurrence_portions_long_decode_and_state(so):
     ts, to, es, er, ec = entries([(1, n)], 2)
     one = so.gated_recurrence(dev(r), dev(i), dev(u), dev(y), lam.cuda(), 8.0, whole, es, er, ec)
     assert torch.equal(one.cpu(), torch.from_numpy(np.concatenate(got))) and torch.equal(whole[1], state[1])
+
+
+@pytest.mark.parametrize("R,H,window,nsplit", [(64, 3, 37, 1), (64, 1, 64, 3), (128, 5, 130, 1), (96, 2, 0, 4), (256, 4, 65, 2), (512, 2, 200, 1), (32, 7, 33, None)])
+def test_latent_window_attn_on_the_matrix_cores(so, R, H, window, nsplit):
+    """the same edges, page borders and far keys through the matrix-core kernel: two portions of two slots and single rows,
+    with and without a split key walk, against the float64 restatement (bf16 operands: tolerance of their rounding)"""
+    rng = np.random.default_rng(R + window + H)
+    n = 330
+    rows = rng.normal(0, 0.3, (n, R)).astype(np.float32)
+    qdir = rng.normal(0, 1, R).astype(np.float32)
+    qdir /= np.linalg.norm(qdir)
+    spikes = [0, 31, 32, 63, 64, 130, 255]
+    for j in spikes:
+        rows[j] = 3.0 * qdir + rng.normal(0, 0.05, R)
+    rows = torch.from_numpy(rows).to(torch.bfloat16).float().numpy()
+    st, tab, slot = filled_cache(rows, torch.bfloat16)
+    assert so.latent_attn_mc_supported(tab)
+    sink = bf(rng.normal(0, 1, H))
+    w = window or n
+    for start, count in ((0, 70), (60, 150), (200, 130), (129, 1), (n - 1, 1), (0, 1), (spikes[3] + w - 1, 2)):
+        if start + count > n:
+            continue
+        pos = list(range(start, start + count))
+        q = (rng.normal(0, 0.2, (count, H * R)) + np.tile(4.0 * qdir, H)).astype(np.float32)
+        qr = torch.from_numpy(q).to(torch.bfloat16).float().numpy()
+        want = attn_ref(qr, rows, pos, H, window, 0.5, sink.float().numpy())
+        i32 = lambda a: torch.tensor(a, dtype=torch.int32).cuda()
+        got = so.latent_window_attn_mc(dev(q), tab, sink.cuda(), i32(pos), i32([slot.index]), i32([0]), i32([count]), count, pos[-1], H, window,
+                                       0.5, nsplit=nsplit)
+        assert rel_err(got.cpu().numpy(), want) < 6e-3, (start, count)     # P is rounded to bf16 for the second product
+        exact = so.latent_window_attn(dev(qr), tab, sink.cuda(), torch.full((count,), slot.index, dtype=torch.int32).cuda(), i32(pos), H, window, 0.5)
+        assert rel_err(got.cpu().numpy(), exact.cpu().numpy()) < 6e-3
+        if window:
+            shifted = attn_ref(qr, rows, pos, H, window + 1, 0.5, sink.float().numpy())
+            if rel_err(shifted, want) > 0.05:
+                assert rel_err(got.cpu().numpy(), shifted) > 0.03
