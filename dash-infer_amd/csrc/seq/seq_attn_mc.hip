@@ -72,7 +72,15 @@ __global__ __launch_bounds__(256) void latent_attn_mc_kernel(McArgs a) {
 #pragma unroll
   for (int t = 0; t < DT; ++t) oacc[t] = z4;
 
-  void* const* tab = a.spans + (size_t)a.ent_slot[e] * a.span_stride;
+  // the span pointers of the walk, staged once: a tile's loads then depend on nothing that is still in flight
+  __shared__ const char* tabs[128];
+  void* const* gtab = a.spans + (size_t)a.ent_slot[e] * a.span_stride;
+  const int span_lo = (my_lo * 32) / a.span_len;
+  for (int i = tid; i < 128; i += 256) {
+    const int sp = span_lo + i;
+    tabs[i] = (sp * a.span_len <= p_hi) ? (const char*)gtab[sp] : nullptr;
+  }
+  __syncthreads();
   const int upr = R >> 3;  // 16-byte units per cached row
   u32x4_t pre[UN];
   auto fetch = [&](int tile) {
@@ -82,7 +90,9 @@ __global__ __launch_bounds__(256) void latent_attn_mc_kernel(McArgs a) {
       pre[j] = u32x4_t{0u, 0u, 0u, 0u};
       if (kin < 32) {
         const int key = tile * 32 + kin;
-        const char* src = (const char*)tab[key / a.span_len] + ((size_t)(key % a.span_len) * R + c8 * 8) * 2;
+        const int sp = key / a.span_len;
+        const char* sb = sp - span_lo < 128 ? tabs[sp - span_lo] : (const char*)gtab[sp];
+        const char* src = sb + ((size_t)(key - sp * a.span_len) * R + c8 * 8) * 2;
         pre[j] = gload<u32x4_t>(src);
       }
     }
@@ -168,19 +178,39 @@ __global__ __launch_bounds__(256) void latent_attn_mc_kernel(McArgs a) {
   }
 }
 
-__global__ __launch_bounds__(64) void latent_attn_merge_kernel(float* __restrict__ out, long ldo, const float* __restrict__ ws, int nsplit,
-                                                               int rows_total, int H, int R) {
+__global__ __launch_bounds__(256) void latent_attn_merge_kernel(float* __restrict__ out, long ldo, const float* __restrict__ ws, int nsplit,
+                                                                int rows_total, int H, int R) {
+  __shared__ float wgt[1024];
+  __shared__ float red[4];
   const int g = blockIdx.x, t = g / H, h = g - t * H;
   const size_t rec = (size_t)R + 4, stride = (size_t)rows_total * rec;
   const float* base = ws + (size_t)g * rec;
-  float mx = -INFINITY;
-  for (int s = 0; s < nsplit; ++s) mx = fmaxf(mx, base[s * stride + R]);
+  float mloc[4], lloc[4], mx = -INFINITY;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int s = threadIdx.x + i * 256;
+    mloc[i] = s < nsplit ? base[s * stride + R] : -INFINITY;
+    lloc[i] = s < nsplit ? base[s * stride + R + 1] : 0.f;
+    mx = fmaxf(mx, mloc[i]);
+  }
+  mx = wave_max(mx);
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = mx;
+  __syncthreads();
+  mx = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
   float den = 0.f;
-  for (int s = 0; s < nsplit; ++s) den += expf(base[s * stride + R] - mx) * base[s * stride + R + 1];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int s = threadIdx.x + i * 256;
+    const float w = s < nsplit ? expf(mloc[i] - mx) : 0.f;
+    if (s < nsplit) wgt[s] = w;
+    den = __builtin_fmaf(w, lloc[i], den);
+  }
+  den = block256_sum(den, red);      // (its barriers publish wgt)
   const float inv = 1.f / den;
-  for (int r = threadIdx.x; r < R; r += 64) {
+  for (int r = threadIdx.x; r < R; r += 256) {
     float acc = 0.f;
-    for (int s = 0; s < nsplit; ++s) acc = __builtin_fmaf(expf(base[s * stride + R] - mx), base[s * stride + r], acc);
+#pragma unroll 8
+    for (int s = 0; s < nsplit; ++s) acc = __builtin_fmaf(wgt[s], base[s * stride + r], acc);
     out[(size_t)t * ldo + (size_t)h * R + r] = acc * inv;
   }
 }
@@ -224,7 +254,7 @@ int dihip_latent_window_attn_mc(void* stream, float* out, long ldo, const float*
   else if (R <= 128) hipLaunchKernelGGL(latent_attn_mc_kernel<128>, grid, dim3(256), lds, s, a);
   else if (R <= 256) hipLaunchKernelGGL(latent_attn_mc_kernel<256>, grid, dim3(256), lds, s, a);
   else hipLaunchKernelGGL(latent_attn_mc_kernel<512>, grid, dim3(256), lds, s, a);
-  if (nsplit > 1) hipLaunchKernelGGL(latent_attn_merge_kernel, dim3(T * H), dim3(64), 0, s, out, ldo, (const float*)ws, nsplit, T * H, H, R);
+  if (nsplit > 1) hipLaunchKernelGGL(latent_attn_merge_kernel, dim3(T * H), dim3(256), 0, s, out, ldo, (const float*)ws, nsplit, T * H, H, R);
   return launch_status();
 }
 

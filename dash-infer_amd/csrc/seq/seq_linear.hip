@@ -176,45 +176,104 @@ __device__ __forceinline__ float dot8_bf16(const u32x4_t& w, const u32x4_t& x, f
   return acc;
 }
 
-// rows t0 .. t0 + tc (tc <= 4) of x staged as bf16 in LDS; wave w of block b owns weight rows (b * 4 + w) * 4 .. + 4.
+// rows t0 .. t0 + tc (tc <= 4) of x staged in LDS -- as bf16, or as they are (EXACT: f32 products of the unrounded row) --;
+// wave w of block b owns weight rows (b * 4 + w) * 2 .. + 2 and keeps two 1 KiB slices of each in flight.
 // K % 8 == 0 and 16-byte aligned weight rows (host-checked).
-template <int XT>
+template <int XT, bool EXACT>
 __global__ __launch_bounds__(256) void linear_skinny_kernel(LinArgs a, int t0, int tc) {
-  extern __shared__ __attribute__((aligned(16))) uint16_t xsm[];
+  extern __shared__ __attribute__((aligned(16))) unsigned char xraw[];
+  uint16_t* xsm = reinterpret_cast<uint16_t*>(xraw);
+  float* xsf = reinterpret_cast<float*>(xraw);
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int g = blockIdx.y;
   const size_t xoff = (size_t)(g % a.xgroups) * a.xg;
-  for (int idx = tid; idx < tc * a.K; idx += 256) {
-    const int t = idx / a.K, k = idx - t * a.K;
-    xsm[idx] = (uint16_t)f32_to_bf16_bits(load_ft<XT>(a.x, (size_t)(t0 + t) * a.ldx + xoff + k));
+  const int nb = (blockIdx.x * 4 + wave) * 2;
+  const bool mine = nb < a.N;
+  const uint16_t* wp = (const uint16_t*)a.w + (size_t)g * a.N * a.K;
+  const uint16_t* w0 = wp + (size_t)min(nb, a.N - 1) * a.K;
+  const uint16_t* w1 = wp + (size_t)min(nb + 1, a.N - 1) * a.K;
+  const u32x4_t z = {0u, 0u, 0u, 0u};
+  u32x4_t cur[2][2], nxt[2][2];
+  auto wload = [&](u32x4_t (&d)[2][2], int k) {   // two 1 KiB slices of both rows, zeros beyond K
+    const bool one = k < a.K, two = k + 512 < a.K;
+    d[0][0] = one ? *reinterpret_cast<const u32x4_t*>(w0 + k) : z;
+    d[1][0] = one ? *reinterpret_cast<const u32x4_t*>(w1 + k) : z;
+    d[0][1] = two ? *reinterpret_cast<const u32x4_t*>(w0 + k + 512) : z;
+    d[1][1] = two ? *reinterpret_cast<const u32x4_t*>(w1 + k + 512) : z;
+  };
+  wload(cur, lane * 8);     // in flight while the rows are staged
+  // staging in units of 8 elements (K % 8 == 0, 16-byte aligned rows: host-checked), several units of a thread in flight
+  const int upr = a.K >> 3, units = tc * upr;
+#pragma unroll 4
+  for (int u = tid; u < units; u += 256) {
+    const int t = u / upr, k = (u - t * upr) * 8;
+    const size_t src = (size_t)(t0 + t) * a.ldx + xoff + k;
+    float v[8];
+    if constexpr (XT == DIHIP_F32) {
+      const f32x4_t lo = *reinterpret_cast<const f32x4_t*>((const float*)a.x + src);
+      const f32x4_t hi = *reinterpret_cast<const f32x4_t*>((const float*)a.x + src + 4);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) { v[j] = lo[j]; v[4 + j] = hi[j]; }
+    } else {
+      const u32x4_t r = *reinterpret_cast<const u32x4_t*>((const uint16_t*)a.x + src);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) { v[2 * j] = __uint_as_float(r[j] << 16); v[2 * j + 1] = __uint_as_float(r[j] & 0xffff0000u); }
+    }
+    if constexpr (EXACT) {
+      *reinterpret_cast<f32x4_t*>(xsf + (size_t)t * a.K + k) = f32x4_t{v[0], v[1], v[2], v[3]};
+      *reinterpret_cast<f32x4_t*>(xsf + (size_t)t * a.K + k + 4) = f32x4_t{v[4], v[5], v[6], v[7]};
+    } else {
+      *reinterpret_cast<u32x4_t*>(xsm + (size_t)t * a.K + k) =
+          u32x4_t{pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]), pack_bf16x2(v[4], v[5]), pack_bf16x2(v[6], v[7])};
+    }
   }
   __syncthreads();
-  const int nb = (blockIdx.x * 4 + wave) * 4;
-  if (nb >= a.N) return;
-  const uint16_t* wp = (const uint16_t*)a.w + (size_t)g * a.N * a.K;
-  float acc[4][4];
+  if (!mine) return;
+  float acc[2][4];
 #pragma unroll
-  for (int i = 0; i < 4; ++i)
+  for (int i = 0; i < 2; ++i)
 #pragma unroll
     for (int t = 0; t < 4; ++t) acc[i][t] = 0.f;
-  for (int k = lane * 8; k < a.K; k += 512) {
-    u32x4_t wv[4];
+  for (int k = lane * 8; k < a.K; k += 1024) {
+    wload(nxt, k + 1024);
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int n = min(nb + i, a.N - 1);
-      wv[i] = *reinterpret_cast<const u32x4_t*>(wp + (size_t)n * a.K + k);
-    }
+    for (int h = 0; h < 2; ++h) {
+      const int kk = k + h * 512;
+      if (kk >= a.K) break;
 #pragma unroll
-    for (int t = 0; t < 4; ++t) {
-      if (t < tc) {
-        const u32x4_t xv = *reinterpret_cast<const u32x4_t*>(xsm + (size_t)t * a.K + k);
+      for (int t = 0; t < 4; ++t) {
+        if (t < tc) {
+          if constexpr (EXACT) {
+            const f32x4_t lo = *reinterpret_cast<const f32x4_t*>(xsf + (size_t)t * a.K + kk);
+            const f32x4_t hi = *reinterpret_cast<const f32x4_t*>(xsf + (size_t)t * a.K + kk + 4);
 #pragma unroll
-        for (int i = 0; i < 4; ++i) acc[i][t] = dot8_bf16(wv[i], xv, acc[i][t]);
+            for (int i = 0; i < 2; ++i) {
+              float v = acc[i][t];
+              v = __builtin_fmaf(__uint_as_float(cur[i][h][0] << 16), lo[0], v);
+              v = __builtin_fmaf(__uint_as_float(cur[i][h][0] & 0xffff0000u), lo[1], v);
+              v = __builtin_fmaf(__uint_as_float(cur[i][h][1] << 16), lo[2], v);
+              v = __builtin_fmaf(__uint_as_float(cur[i][h][1] & 0xffff0000u), lo[3], v);
+              v = __builtin_fmaf(__uint_as_float(cur[i][h][2] << 16), hi[0], v);
+              v = __builtin_fmaf(__uint_as_float(cur[i][h][2] & 0xffff0000u), hi[1], v);
+              v = __builtin_fmaf(__uint_as_float(cur[i][h][3] << 16), hi[2], v);
+              v = __builtin_fmaf(__uint_as_float(cur[i][h][3] & 0xffff0000u), hi[3], v);
+              acc[i][t] = v;
+            }
+          } else {
+            const u32x4_t xv = *reinterpret_cast<const u32x4_t*>(xsm + (size_t)t * a.K + kk);
+#pragma unroll
+            for (int i = 0; i < 2; ++i) acc[i][t] = dot8_bf16(cur[i][h], xv, acc[i][t]);
+          }
+        }
       }
     }
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int h = 0; h < 2; ++h) cur[i][h] = nxt[i][h];
   }
 #pragma unroll
-  for (int i = 0; i < 4; ++i)
+  for (int i = 0; i < 2; ++i)
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
       const float v = wave_sum(acc[i][t]);
@@ -236,7 +295,8 @@ extern "C" int dihip_linear(void* stream, const void* x, int x_dtype, long ldx, 
   DIHIP_REQUIRE(seq_dtype_ok(x_dtype) && seq_dtype_ok(w_dtype) && seq_dtype_ok(y_dtype), DIHIP_PARAM_ERROR, "linear: f32 / bf16 only");
   DIHIP_REQUIRE(x && w && y, DIHIP_PARAM_ERROR, "linear: null pointer");
   DIHIP_REQUIRE(ldx >= K && ldy >= N && (!mul || ldm >= N), DIHIP_PARAM_ERROR, "linear: a row stride below the row length");
-  DIHIP_REQUIRE(math == DIHIP_MATH_F32 || math == DIHIP_MATH_BF16, DIHIP_PARAM_ERROR, "linear: unknown math mode %d", math);
+  DIHIP_REQUIRE(math == DIHIP_MATH_F32 || math == DIHIP_MATH_BF16 || math == DIHIP_MATH_F32_STREAM, DIHIP_PARAM_ERROR,
+                "linear: unknown math mode %d", math);
   DIHIP_REQUIRE(groups <= 65535, DIHIP_PARAM_ERROR, "linear: more than 65535 groups");
   if (T == 0) return DIHIP_SUCCESS;
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
@@ -244,15 +304,29 @@ extern "C" int dihip_linear(void* stream, const void* x, int x_dtype, long ldx, 
   const size_t xe = x_dtype == DIHIP_F32 ? 4 : 2;
   const bool vec = w_dtype == DIHIP_BF16 && K % 8 == 0 && aligned16(w) && aligned16(x) && (ldx * xe) % 16 == 0 &&
                    (x_gstride * xe) % 16 == 0;
+  static const bool no_skinny = env_off("DIHIP_LINEAR_SKINNY");
+  if (math == DIHIP_MATH_F32_STREAM) {
+    // f32 products of unrounded rows; few rows stream the weight once (a row's sum then runs in the lanes' order, not k ascending)
+    const int tmax = K <= 4096 ? 4 : (K <= 8192 ? 2 : 1);
+    if (T <= 4 * tmax && vec && !no_skinny && K <= 16384) {
+      for (int t0 = 0; t0 < T; t0 += tmax) {
+        const int tc = T - t0 < tmax ? T - t0 : tmax;
+        const dim3 grid((N + 7) / 8, groups);
+        if (x_dtype == DIHIP_F32) hipLaunchKernelGGL((linear_skinny_kernel<DIHIP_F32, true>), grid, dim3(256), (size_t)tc * K * 4, s, a, t0, tc);
+        else hipLaunchKernelGGL((linear_skinny_kernel<DIHIP_BF16, true>), grid, dim3(256), (size_t)tc * K * 4, s, a, t0, tc);
+      }
+      return launch_status();
+    }
+    math = DIHIP_MATH_F32;
+  }
   if (math == DIHIP_MATH_BF16 && w_dtype == DIHIP_BF16) {
-    static const bool no_skinny = env_off("DIHIP_LINEAR_SKINNY");
     const int tmax = K <= 8192 ? 4 : (K <= 16384 ? 2 : 1);  // rows whose bf16 copy fits 64 KB of LDS
     if (T <= 4 * tmax && vec && !no_skinny && K <= 32768) {
       for (int t0 = 0; t0 < T; t0 += tmax) {
         const int tc = T - t0 < tmax ? T - t0 : tmax;
-        const dim3 grid((N + 15) / 16, groups);
-        if (x_dtype == DIHIP_F32) hipLaunchKernelGGL(linear_skinny_kernel<DIHIP_F32>, grid, dim3(256), (size_t)tc * K * 2, s, a, t0, tc);
-        else hipLaunchKernelGGL(linear_skinny_kernel<DIHIP_BF16>, grid, dim3(256), (size_t)tc * K * 2, s, a, t0, tc);
+        const dim3 grid((N + 7) / 8, groups);
+        if (x_dtype == DIHIP_F32) hipLaunchKernelGGL((linear_skinny_kernel<DIHIP_F32, false>), grid, dim3(256), (size_t)tc * K * 2, s, a, t0, tc);
+        else hipLaunchKernelGGL((linear_skinny_kernel<DIHIP_BF16, false>), grid, dim3(256), (size_t)tc * K * 2, s, a, t0, tc);
       }
       return launch_status();
     }

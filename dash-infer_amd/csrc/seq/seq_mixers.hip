@@ -11,13 +11,16 @@ namespace dihip {
 namespace {
 
 // ------------------------------------------------------------------------------------------------ embedding
+template <int WT>
 __global__ __launch_bounds__(256) void embed_sum_kernel(float* __restrict__ h, const int32_t* __restrict__ ids, const void* __restrict__ table,
-                                                        const int32_t* __restrict__ rows2, const void* __restrict__ table2, int wdt, int K) {
+                                                        const int32_t* __restrict__ rows2, const void* __restrict__ table2, int K) {
   const int t = blockIdx.x;
   const size_t r1 = (size_t)ids[t] * K, r2 = table2 ? (size_t)rows2[t] * K : 0;
+  const bool two = table2 != nullptr;
+#pragma unroll 4
   for (int k = threadIdx.x; k < K; k += 256) {
-    float v = ld_any(table, r1 + k, wdt);
-    if (table2) v += ld_any(table2, r2 + k, wdt);
+    float v = load_ft<WT>(table, r1 + k);
+    if (two) v += load_ft<WT>(table2, r2 + k);
     h[(size_t)t * K + k] = v;
   }
 }
@@ -26,25 +29,40 @@ __global__ __launch_bounds__(256) void embed_sum_kernel(float* __restrict__ h, c
 // sum of squares of a row, k ascending per thread, one fixed tree over the block
 __device__ __forceinline__ float row_sumsq(const float* __restrict__ x, int K, float* red) {
   float ss = 0.f;
-  for (int k = threadIdx.x; k < K; k += 256) {
-    const float v = x[k];
-    ss = __builtin_fmaf(v, v, ss);
+  if ((K & 3) == 0 && (reinterpret_cast<uintptr_t>(x) & 15u) == 0) {   // (block-uniform) 16-byte loads, four of them in flight
+#pragma unroll 4
+    for (int k = threadIdx.x * 4; k < K; k += 1024) {
+      const f32x4_t v = *reinterpret_cast<const f32x4_t*>(x + k);
+      ss = __builtin_fmaf(v[0], v[0], ss);
+      ss = __builtin_fmaf(v[1], v[1], ss);
+      ss = __builtin_fmaf(v[2], v[2], ss);
+      ss = __builtin_fmaf(v[3], v[3], ss);
+    }
+  } else {
+#pragma unroll 8
+    for (int k = threadIdx.x; k < K; k += 256) {
+      const float v = x[k];
+      ss = __builtin_fmaf(v, v, ss);
+    }
   }
   return block256_sum(ss, red);
 }
 
+template <int WT>
 __global__ __launch_bounds__(256) void rmsnorm_strided_kernel(void* __restrict__ y, int ydt, long ldy, const float* __restrict__ x, long ldx,
-                                                              const int32_t* __restrict__ row_idx, const void* __restrict__ gamma, int wdt,
+                                                              const int32_t* __restrict__ row_idx, const void* __restrict__ gamma,
                                                               float eps, int K) {
   __shared__ float red[4];
   const int i = blockIdx.x;
   const float* xr = x + (size_t)(row_idx ? row_idx[i] : i) * ldx;
   const float inv = 1.f / sqrtf(row_sumsq(xr, K, red) / (float)K + eps);
-  for (int k = threadIdx.x; k < K; k += 256) st_any(y, (size_t)i * ldy + k, ydt, xr[k] * inv * ld_any(gamma, k, wdt));
+#pragma unroll 4
+  for (int k = threadIdx.x; k < K; k += 256) st_any(y, (size_t)i * ldy + k, ydt, xr[k] * inv * load_ft<WT>(gamma, k));
 }
 
+template <int WT>
 __global__ __launch_bounds__(256) void norm_span_append_kernel(void* const* __restrict__ spans, int span_stride, int span_len, int cdt,
-                                                               const float* __restrict__ x, long ldx, const void* __restrict__ gamma, int wdt,
+                                                               const float* __restrict__ x, long ldx, const void* __restrict__ gamma,
                                                                float eps, const int32_t* __restrict__ tok_slot,
                                                                const int32_t* __restrict__ tok_pos, int K) {
   __shared__ float red[4];
@@ -54,26 +72,46 @@ __global__ __launch_bounds__(256) void norm_span_append_kernel(void* const* __re
   const int pos = tok_pos[t];
   void* span = spans[(size_t)tok_slot[t] * span_stride + pos / span_len];
   const size_t base = (size_t)(pos % span_len) * K;
-  for (int k = threadIdx.x; k < K; k += 256) st_any(span, base + k, cdt, xr[k] * inv * ld_any(gamma, k, wdt));
+#pragma unroll 4
+  for (int k = threadIdx.x; k < K; k += 256) st_any(span, base + k, cdt, xr[k] * inv * load_ft<WT>(gamma, k));
 }
 
+// The depth mix reads every earlier level of the stack: its weights are staged in LDS and the levels are read through a
+// restrict view (the level written here is never one of them), so that a thread's loads are all in flight together.
+template <int WT>
 __global__ __launch_bounds__(256) void norm_residual_mix_kernel(float* x_out, const float* x_in, const float* __restrict__ m,
-                                                                long ldm, const void* __restrict__ gamma, int wdt, float eps,
-                                                                float* __restrict__ stack, size_t stack_stride, const void* __restrict__ mix_w,
-                                                                int n_mix, float* __restrict__ x_mix, int K) {
+                                                                long ldm, const void* __restrict__ gamma, float eps,
+                                                                float* stack_top, const float* __restrict__ stack, size_t stack_stride,
+                                                                const void* __restrict__ mix_w, int n_mix, float* __restrict__ x_mix, int K) {
   __shared__ float red[4];
+  __shared__ float mw[256];
   const int t = blockIdx.x;
+  if (threadIdx.x < n_mix) mw[threadIdx.x] = load_ft<WT>(mix_w, threadIdx.x);
   const float* mr = m + (size_t)t * ldm;
-  const float inv = 1.f / sqrtf(row_sumsq(mr, K, red) / (float)K + eps);
+  const float inv = 1.f / sqrtf(row_sumsq(mr, K, red) / (float)K + eps);   // (its barriers publish mw)
   const size_t row = (size_t)t * K;
-  for (int k = threadIdx.x; k < K; k += 256) {
-    const float xo = x_in[row + k] + mr[k] * inv * ld_any(gamma, k, wdt);
-    x_out[row + k] = xo;
-    if (n_mix > 0) {
-      stack[(size_t)(n_mix - 1) * stack_stride + row + k] = xo;
-      float mix = 0.f;
-      for (int j = 0; j + 1 < n_mix; ++j) mix = __builtin_fmaf(ld_any(mix_w, j, wdt), stack[(size_t)j * stack_stride + row + k], mix);
-      x_mix[row + k] = __builtin_fmaf(ld_any(mix_w, n_mix - 1, wdt), xo, mix);
+  for (int k0 = threadIdx.x; k0 < K; k0 += 1024) {
+    float xo[4], mix[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int k = k0 + i * 256;
+      xo[i] = mix[i] = 0.f;
+      if (k < K) {
+        xo[i] = x_in[row + k] + mr[k] * inv * load_ft<WT>(gamma, k);
+#pragma unroll 4
+        for (int j = 0; j + 1 < n_mix; ++j) mix[i] = __builtin_fmaf(mw[j], stack[(size_t)j * stack_stride + row + k], mix[i]);
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int k = k0 + i * 256;
+      if (k < K) {
+        x_out[row + k] = xo[i];
+        if (n_mix > 0) {
+          stack_top[row + k] = xo[i];
+          x_mix[row + k] = __builtin_fmaf(mw[n_mix - 1], xo[i], mix[i]);
+        }
+      }
     }
   }
 }
@@ -233,6 +271,66 @@ __global__ __launch_bounds__(64) void gated_recurrence_kernel(float* __restrict_
   *sp = S;
 }
 
+// Long portions: the recurrence S_t = a_t S_(t-1) + g_t is a composition of affine maps, so a portion is cut into chunks of
+// REC_CHUNK rows that run side by side.  Pass 1: every (chunk, channel) composes its rows from S = 0: (A = prod a_t, B = the
+// state it would end in).  Pass 2 (per channel, chunks in order): the state each chunk really starts from, S <- A S + B.
+// Pass 3: every chunk runs its rows from that state and writes the outputs.  The cut changes the result by f32 rounding only.
+constexpr int REC_CHUNK = 64;
+
+struct RecArgs {
+  float* out; long ldo; const float* r; const float* ig; long ldg; const float* u; long ldu; const float* y; long ldy;
+  const void* lam; int wdt; float decay; float* state; const int32_t* ent_slot; const int32_t* ent_row0; const int32_t* ent_count;
+  int C; float* ab; int max_chunks;   // ab: [E][max_chunks][2][C]
+};
+
+template <int PASS>
+__global__ __launch_bounds__(64) void gated_recurrence_chunk_kernel(RecArgs a) {
+  const int e = blockIdx.z, ch = blockIdx.x, c = blockIdx.y * 64 + threadIdx.x;
+  const int cnt = a.ent_count[e], row0 = a.ent_row0[e];
+  const int lo = ch * REC_CHUNK;
+  if (c >= a.C || lo >= cnt) return;
+  const int n = min(REC_CHUNK, cnt - lo);
+  float* ab = a.ab + ((size_t)e * a.max_chunks + ch) * 2 * a.C;
+  const float k = -a.decay * softplus_f32(ld_any(a.lam, c, a.wdt));
+  float S = PASS == 1 ? 0.f : ab[c], A = 1.f;
+  constexpr int U = 8;
+  for (int i0 = 0; i0 < n; i0 += U) {
+    float rv[U], iv[U], uv[U], yv[U];
+#pragma unroll
+    for (int j = 0; j < U; ++j) {
+      const size_t t = (size_t)(row0 + lo + min(i0 + j, n - 1));
+      rv[j] = a.r[t * a.ldg + c]; iv[j] = a.ig[t * a.ldg + c]; uv[j] = a.u[t * a.ldu + c];
+      if (PASS == 3) yv[j] = a.y[t * a.ldy + c];
+    }
+#pragma unroll
+    for (int j = 0; j < U; ++j) {
+      if (i0 + j < n) {
+        const float la = k * rv[j];
+        const float av = expf(la);
+        S = __builtin_fmaf(av, S, sqrtf(-expm1f(2.f * la)) * iv[j] * uv[j]);
+        if (PASS == 1) A *= av;
+        else a.out[(size_t)(row0 + lo + i0 + j) * a.ldo + c] = S * yv[j];
+      }
+    }
+  }
+  if (PASS == 1) { ab[c] = A; ab[a.C + c] = S; }
+  else if (lo + n == cnt) a.state[(size_t)a.ent_slot[e] * a.C + c] = S;
+}
+
+// pass 2: ab[ch][0] <- the state chunk ch starts from
+__global__ __launch_bounds__(64) void gated_recurrence_carry_kernel(RecArgs a) {
+  const int e = blockIdx.x, c = blockIdx.y * 64 + threadIdx.x;
+  if (c >= a.C) return;
+  const int chunks = (a.ent_count[e] + REC_CHUNK - 1) / REC_CHUNK;
+  float S = a.state[(size_t)a.ent_slot[e] * a.C + c];
+  for (int ch = 0; ch < chunks; ++ch) {
+    float* ab = a.ab + ((size_t)e * a.max_chunks + ch) * 2 * a.C;
+    const float A = ab[c], B = ab[a.C + c];
+    ab[c] = S;
+    S = __builtin_fmaf(A, S, B);
+  }
+}
+
 static thread_local char g_seq_error[512] = "";
 
 }  // namespace
@@ -265,7 +363,8 @@ int dihip_embed_sum(void* stream, float* h, const int32_t* ids, const void* tabl
                     int w_dtype, int T, int K) {
   DIHIP_REQUIRE(T >= 0 && K > 0 && h && ids && table && (!table2 || rows2) && seq_dtype_ok(w_dtype), DIHIP_PARAM_ERROR, "embed_sum: bad argument");
   if (T == 0) return DIHIP_SUCCESS;
-  hipLaunchKernelGGL(embed_sum_kernel, dim3(T), dim3(256), 0, reinterpret_cast<hipStream_t>(stream), h, ids, table, rows2, table2, w_dtype, K);
+  if (w_dtype == DIHIP_F32) hipLaunchKernelGGL(embed_sum_kernel<DIHIP_F32>, dim3(T), dim3(256), 0, reinterpret_cast<hipStream_t>(stream), h, ids, table, rows2, table2, K);
+  else hipLaunchKernelGGL(embed_sum_kernel<DIHIP_BF16>, dim3(T), dim3(256), 0, reinterpret_cast<hipStream_t>(stream), h, ids, table, rows2, table2, K);
   return launch_status();
 }
 
@@ -274,8 +373,8 @@ int dihip_rmsnorm_strided(void* stream, void* y, int y_dtype, long ldy, const fl
   DIHIP_REQUIRE(M >= 0 && K > 0 && y && x && gamma && ldy >= K && ldx >= K && seq_dtype_ok(y_dtype) && seq_dtype_ok(w_dtype),
                 DIHIP_PARAM_ERROR, "rmsnorm_strided: bad argument");
   if (M == 0) return DIHIP_SUCCESS;
-  hipLaunchKernelGGL(rmsnorm_strided_kernel, dim3(M), dim3(256), 0, reinterpret_cast<hipStream_t>(stream), y, y_dtype, ldy, x, ldx, row_idx,
-                     gamma, w_dtype, eps, K);
+  if (w_dtype == DIHIP_F32) hipLaunchKernelGGL(rmsnorm_strided_kernel<DIHIP_F32>, dim3(M), dim3(256), 0, reinterpret_cast<hipStream_t>(stream), y, y_dtype, ldy, x, ldx, row_idx, gamma, eps, K);
+  else hipLaunchKernelGGL(rmsnorm_strided_kernel<DIHIP_BF16>, dim3(M), dim3(256), 0, reinterpret_cast<hipStream_t>(stream), y, y_dtype, ldy, x, ldx, row_idx, gamma, eps, K);
   return launch_status();
 }
 
@@ -284,8 +383,8 @@ int dihip_norm_span_append(void* stream, void* const* spans, int span_stride, in
   DIHIP_REQUIRE(T >= 0 && K > 0 && spans && x && gamma && tok_slot && tok_pos && span_stride > 0 && span_len > 0 && ldx >= K &&
                     seq_dtype_ok(cache_dtype) && seq_dtype_ok(w_dtype), DIHIP_PARAM_ERROR, "norm_span_append: bad argument");
   if (T == 0) return DIHIP_SUCCESS;
-  hipLaunchKernelGGL(norm_span_append_kernel, dim3(T), dim3(256), 0, reinterpret_cast<hipStream_t>(stream), spans, span_stride, span_len,
-                     cache_dtype, x, ldx, gamma, w_dtype, eps, tok_slot, tok_pos, K);
+  if (w_dtype == DIHIP_F32) hipLaunchKernelGGL(norm_span_append_kernel<DIHIP_F32>, dim3(T), dim3(256), 0, reinterpret_cast<hipStream_t>(stream), spans, span_stride, span_len, cache_dtype, x, ldx, gamma, eps, tok_slot, tok_pos, K);
+  else hipLaunchKernelGGL(norm_span_append_kernel<DIHIP_BF16>, dim3(T), dim3(256), 0, reinterpret_cast<hipStream_t>(stream), spans, span_stride, span_len, cache_dtype, x, ldx, gamma, eps, tok_slot, tok_pos, K);
   return launch_status();
 }
 
@@ -296,8 +395,10 @@ int dihip_norm_residual_mix(void* stream, float* x_out, const float* x_in, const
   DIHIP_REQUIRE(n_mix == 0 || (stack && mix_w && x_mix && stack_stride >= (size_t)T * K && x_mix != x_out), DIHIP_PARAM_ERROR,
                 "norm_residual_mix: the depth mix needs the stack, its weights and an output of its own");
   if (T == 0) return DIHIP_SUCCESS;
-  hipLaunchKernelGGL(norm_residual_mix_kernel, dim3(T), dim3(256), 0, reinterpret_cast<hipStream_t>(stream), x_out, x_in, m, ldm, gamma,
-                     w_dtype, eps, stack, stack_stride, mix_w, n_mix, x_mix, K);
+  DIHIP_REQUIRE(n_mix <= 256, DIHIP_EXCEED_LIMIT_ERROR, "norm_residual_mix: more than 256 levels");
+  float* top = n_mix > 0 ? stack + (size_t)(n_mix - 1) * stack_stride : nullptr;
+  if (w_dtype == DIHIP_F32) hipLaunchKernelGGL(norm_residual_mix_kernel<DIHIP_F32>, dim3(T), dim3(256), 0, reinterpret_cast<hipStream_t>(stream), x_out, x_in, m, ldm, gamma, eps, top, stack, stack_stride, mix_w, n_mix, x_mix, K);
+  else hipLaunchKernelGGL(norm_residual_mix_kernel<DIHIP_BF16>, dim3(T), dim3(256), 0, reinterpret_cast<hipStream_t>(stream), x_out, x_in, m, ldm, gamma, eps, top, stack, stack_stride, mix_w, n_mix, x_mix, K);
   return launch_status();
 }
 
@@ -346,6 +447,30 @@ int dihip_conv_tail_update(void* stream, float* tail, const float* x, long ldx, 
   DIHIP_REQUIRE(tail, DIHIP_PARAM_ERROR, "conv_tail_update: null state");
   hipLaunchKernelGGL(conv_tail_update_kernel, dim3(E, (C + 255) / 256), dim3(256), 0, reinterpret_cast<hipStream_t>(stream), tail, x, ldx,
                      ent_slot, ent_row0, ent_count, C, taps);
+  return launch_status();
+}
+
+size_t dihip_gated_recurrence_chunked_workspace_bytes(int E, int max_count, int C) {
+  return (size_t)E * ((max_count + REC_CHUNK - 1) / REC_CHUNK) * 2 * C * sizeof(float);
+}
+
+int dihip_gated_recurrence_chunked(void* stream, float* out, long ldo, const float* r, const float* i, long ldg, const float* u, long ldu,
+                                   const float* y, long ldy, const void* lam, int w_dtype, float decay, float* state,
+                                   const int32_t* ent_slot, const int32_t* ent_row0, const int32_t* ent_count, int E, int max_count, int C,
+                                   void* ws, size_t ws_bytes) {
+  DIHIP_REQUIRE(E >= 0 && max_count >= 0 && C > 0 && out && r && i && u && y && lam && state && ent_slot && ent_row0 && ent_count &&
+                    ldo >= C && ldg >= C && ldu >= C && ldy >= C && seq_dtype_ok(w_dtype) && E <= 65535, DIHIP_PARAM_ERROR,
+                "gated_recurrence_chunked: bad argument");
+  DIHIP_REQUIRE(ws && ws_bytes >= dihip_gated_recurrence_chunked_workspace_bytes(E, max_count, C), DIHIP_PARAM_ERROR,
+                "gated_recurrence_chunked: workspace too small");
+  if (E == 0 || max_count == 0) return DIHIP_SUCCESS;
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  const int chunks = (max_count + REC_CHUNK - 1) / REC_CHUNK;
+  RecArgs a{out, ldo, r, i, ldg, u, ldu, y, ldy, lam, w_dtype, decay, state, ent_slot, ent_row0, ent_count, C, (float*)ws, chunks};
+  const dim3 grid(chunks, (C + 63) / 64, E);
+  hipLaunchKernelGGL(gated_recurrence_chunk_kernel<1>, grid, dim3(64), 0, s, a);
+  hipLaunchKernelGGL(gated_recurrence_carry_kernel, dim3(E, (C + 63) / 64), dim3(64), 0, s, a);
+  hipLaunchKernelGGL(gated_recurrence_chunk_kernel<3>, grid, dim3(64), 0, s, a);
   return launch_status();
 }
 

@@ -28,6 +28,12 @@ class SeqEngine:
         self.model = model_cls.from_config(config, tensors, self.state, dtype)
         self.vocab = self.model.vocab
         self.state.upload()
+        # decode steps (one token of every request, every one's logits wanted) replay a captured hipGraph per (requests, length
+        # bucket): the launches of a step are fixed once its sizes are, its numbers (tokens, positions, slots) lie in a device
+        # buffer that is refilled before the replay.  DIHIP_SEQ_GRAPH=0: eager launches.
+        import os
+        self.use_graphs = dtype == torch.bfloat16 and os.environ.get("DIHIP_SEQ_GRAPH", "1") != "0"
+        self._graphs = {}
 
     @classmethod
     def from_pretrained(cls, path, dtype=torch.bfloat16, device="cuda", **kw):
@@ -83,21 +89,51 @@ class SeqEngine:
             rows2 = [0] * T
         flat = ids + rows2 + tslot + tpos + toff + eslot + erow0 + ecnt + want
         host = torch.tensor(flat, dtype=torch.int32)
+        cut = [T, T, T, T, T, E, E, E, len(want)]
+        if self.use_graphs and taps is None and T == E and want == list(range(E)):
+            return self._decode_step(host, cut, T, max(tpos))
         if torch.cuda.is_available():
             host = host.pin_memory()
-        dev = host.to(self.device, non_blocking=True)
-        cut = [T, T, T, T, T, E, E, E, len(want)]
-        parts, o = [], 0
-        for n in cut:
-            parts.append(dev[o:o + n])
-            o += n
-        ctx = StepContext(T, E, *parts, math=model.math, eps=model.eps)
+        ctx = self._context(host.to(self.device, non_blocking=True), cut, T, E, max(ecnt), max(tpos))
         ctx.taps = taps
-        ctx.max_count, ctx.max_pos = max(ecnt), max(tpos)
         x = model.forward(ctx)
         if not want:
             return None
         return model.logits(ctx, x, ctx.want_rows)
+
+    def _context(self, dev, cut, T, E, max_count, max_pos):
+        parts, o = [], 0
+        for n in cut:
+            parts.append(dev[o:o + n])
+            o += n
+        ctx = StepContext(T, E, *parts, math=self.model.math, eps=self.model.eps)
+        ctx.max_count, ctx.max_pos = max_count, max_pos
+        return ctx
+
+    def _decode_step(self, host, cut, E, max_pos):
+        """one token of each of E requests: the first step of a (E, length bucket) runs eagerly and is then captured, later ones
+        replay.  The returned logits are the graph's own buffer: valid until the next step."""
+        bucket = (max_pos + 512) // 512 * 512 - 1       # the split of the attention's key walk follows this, not the exact length
+        g = self._graphs.get((E, bucket))
+        if g is None:
+            g = {"host": torch.empty(host.numel(), dtype=torch.int32, pin_memory=True),
+                 "meta": torch.empty(host.numel(), dtype=torch.int32, device=self.device), "graph": None}
+            if len(self._graphs) < 64:
+                self._graphs[(E, bucket)] = g
+        g["host"].copy_(host)
+        g["meta"].copy_(g["host"], non_blocking=True)
+        if g["graph"] is not None:
+            g["graph"].replay()
+            return g["logits"]
+        ctx = self._context(g["meta"], cut, E, E, 1, bucket)
+        logits = self.model.logits(ctx, self.model.forward(ctx), ctx.want_rows)
+        if (E, bucket) in self._graphs:
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):      # records the same launches; nothing runs, the state is not touched
+                g["logits"] = self.model.logits(ctx, self.model.forward(ctx), ctx.want_rows)
+            g["graph"] = graph
+        return logits
 
     def release(self, rid):
         if rid in self.state.live:

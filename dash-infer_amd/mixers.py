@@ -90,8 +90,10 @@ class GatedLinearRecurrence:
         u = so.causal_conv_state(x, self.conv, self.conv_b, self.tail, ctx.tok_slot, ctx.tok_off)
         if self.tail is not None:
             so.conv_tail_update(self.tail, x, self.taps, ctx.ent_slot, ctx.ent_row0, ctx.ent_count)
-        g = so.linear(u, self.w_gate, self.b_gate, act="sigmoid", groups=2 * self.B, x_groups=self.B, math=so.MATH_F32)
-        sy = so.gated_recurrence(g[:, :C], g[:, C:], u, y, self.lam, self.decay, self.S, ctx.ent_slot, ctx.ent_row0, ctx.ent_count)
+        g = so.linear(u, self.w_gate, self.b_gate, act="sigmoid", groups=2 * self.B, x_groups=self.B,
+                      math=so.MATH_F32 if ctx.math == so.MATH_F32 else so.MATH_F32_STREAM)    # f32 products in both engines
+        sy = so.gated_recurrence(g[:, :C], g[:, C:], u, y, self.lam, self.decay, self.S, ctx.ent_slot, ctx.ent_row0, ctx.ent_count,
+                                 max_count=ctx.max_count)
         return so.linear(sy, self.o, math=ctx.math)
 
 

@@ -12,7 +12,7 @@ from . import PKG_DIR
 
 SEQ_LIB_PATH = os.path.join(os.environ.get("DIHIP_LIB_DIR") or os.path.join(PKG_DIR, "lib"), "libdashinfer_hip_seq.so")
 F32, BF16 = 0, 2
-MATH_F32, MATH_BF16 = 0, 1
+MATH_F32, MATH_BF16, MATH_F32_STREAM = 0, 1, 2
 ACT = {None: 0, "none": 0, "tanh": 1, "gelu_erf": 2, "gelu_tanh": 3, "relu": 4, "silu": 5, "sigmoid": 6}
 
 vp, sz, i32, f32, lng = C.c_void_p, C.c_size_t, C.c_int, C.c_float, C.c_long
@@ -32,6 +32,8 @@ _SIGS = {
                                           vp, sz]),
     "dihip_causal_conv_state": (i32, [vp, vp, lng, vp, lng, vp, vp, i32, vp, vp, vp, i32, i32, i32]),
     "dihip_conv_tail_update": (i32, [vp, vp, vp, lng, vp, vp, vp, i32, i32, i32]),
+    "dihip_gated_recurrence_chunked_workspace_bytes": (sz, [i32, i32, i32]),
+    "dihip_gated_recurrence_chunked": (i32, [vp, vp, lng, vp, vp, lng, vp, lng, vp, lng, vp, i32, f32, vp, vp, vp, vp, i32, i32, i32, vp, sz]),
     "dihip_gated_recurrence": (i32, [vp, vp, lng, vp, vp, lng, vp, lng, vp, lng, vp, i32, f32, vp, vp, vp, vp, i32, i32]),
 }
 

@@ -9,7 +9,7 @@ import ctypes as C
 import torch
 
 from . import seq_capi
-from .seq_capi import ACT, MATH_BF16, MATH_F32, check, lib
+from .seq_capi import ACT, MATH_BF16, MATH_F32, MATH_F32_STREAM, check, lib
 
 _DT = {torch.float32: seq_capi.F32, torch.bfloat16: seq_capi.BF16}
 
@@ -110,10 +110,10 @@ def latent_window_attn_mc(q, table, sink, tok_pos, ent_slot, ent_row0, ent_count
     (host numbers: they size the grid and the split of the key walk)"""
     T, R, E = q.shape[0], table.row_elems, ent_slot.shape[0]
     o = out if out is not None else torch.empty(T, H * R, dtype=torch.float32, device=q.device)
-    if nsplit is None:       # fill the chip: ~2 workgroups per CU; at least 4 key tiles (128 keys) per workgroup
+    if nsplit is None:       # fill the chip: ~2 workgroups per CU; at least 2 key tiles (64 keys) per workgroup
         blocks = max(1, E * ((max_count * H + 63) // 64))
         keys = min(max_pos + 1, window) if window > 0 else max_pos + 1
-        nsplit = max(1, min(512 // blocks, (keys + 127) // 128))
+        nsplit = max(1, min(512 // blocks, (keys + 63) // 64))
     ws = None
     if nsplit > 1:
         ws = torch.empty(int(lib().dihip_latent_window_attn_mc_workspace_bytes(T, H, R, nsplit)), dtype=torch.uint8, device=q.device)
@@ -138,10 +138,21 @@ def conv_tail_update(tail, x, taps, ent_slot, ent_row0, ent_count):
                                        ent_slot.shape[0], x.shape[1], taps), "dihip_conv_tail_update")
 
 
-def gated_recurrence(r, i, u, y, lam, decay, state, ent_slot, ent_row0, ent_count, out=None):
+CHUNKED_RECURRENCE_ROWS = 256   # portions from this length on run as chunks side by side
+
+
+def gated_recurrence(r, i, u, y, lam, decay, state, ent_slot, ent_row0, ent_count, out=None, max_count=None):
+    """max_count: the step's largest portion (a host number); given and >= CHUNKED_RECURRENCE_ROWS: the chunk-parallel form"""
     T, Cn = u.shape
     assert _rows(r) == _rows(i)
     o = out if out is not None else torch.empty(T, Cn, dtype=torch.float32, device=u.device)
+    if max_count is not None and max_count >= CHUNKED_RECURRENCE_ROWS:
+        E = ent_slot.shape[0]
+        ws = torch.empty(int(lib().dihip_gated_recurrence_chunked_workspace_bytes(E, max_count, Cn)), dtype=torch.uint8, device=u.device)
+        check(lib().dihip_gated_recurrence_chunked(stream(), ptr(o), _rows(o), ptr(r), ptr(i), _rows(r), ptr(u), _rows(u), ptr(y), _rows(y),
+                                                   ptr(lam), dt(lam), float(decay), ptr(state), ptr(ent_slot), ptr(ent_row0), ptr(ent_count),
+                                                   E, int(max_count), Cn, ptr(ws), ws.numel()), "dihip_gated_recurrence_chunked")
+        return o
     check(lib().dihip_gated_recurrence(stream(), ptr(o), _rows(o), ptr(r), ptr(i), _rows(r), ptr(u), _rows(u), ptr(y), _rows(y), ptr(lam),
                                        dt(lam), float(decay), ptr(state), ptr(ent_slot), ptr(ent_row0), ptr(ent_count),
                                        ent_slot.shape[0], Cn), "dihip_gated_recurrence")

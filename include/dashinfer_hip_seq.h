@@ -27,7 +27,9 @@ const char* dihip_seq_last_error(void);
 
 /* math of dihip_linear: EXACT = every product and sum in f32, k ascending; BF16 = operands rounded to bf16, f32
  * accumulation on the matrix cores (T > DIHIP_LINEAR_SKINNY_ROWS) or in a weight-streaming dot-product kernel */
-enum { DIHIP_MATH_F32 = 0, DIHIP_MATH_BF16 = 1 };
+enum { DIHIP_MATH_F32 = 0, DIHIP_MATH_BF16 = 1, DIHIP_MATH_F32_STREAM = 2 };
+/* F32_STREAM = F32 products of the unrounded operands, but few rows (decoding) stream the weight through the dot-product
+ * kernel, whose sums run in the lanes' order: for the f32 parts of a bf16 engine (gates of a recurrence) */
 
 /* y[g][t, n] = epilogue( sum_k x[g % x_groups][t, k] * w[g][n, k] + bias[g][n] ),  g < groups, t < T, n < N
  *   x: [T, .] rows of stride ldx, group g starts at column (g % x_groups) * x_gstride;  w: [groups][N][K] row-major,
@@ -97,6 +99,14 @@ int dihip_gated_recurrence(void* stream, float* out, long ldo, const float* r, c
                            const float* u, long ldu, const float* y, long ldy, const void* lam, int w_dtype,
                            float decay, float* state, const int32_t* ent_slot, const int32_t* ent_row0,
                            const int32_t* ent_count, int E, int C);
+/* the same recurrence with every portion cut into chunks of 64 rows that run side by side (three launches: compose each
+ * chunk from zero, carry the states over the chunks, run the chunks from their true start states): for long portions.
+ * The result differs from the row-by-row form by f32 rounding only.  max_count = the largest ent_count. */
+size_t dihip_gated_recurrence_chunked_workspace_bytes(int E, int max_count, int C);
+int dihip_gated_recurrence_chunked(void* stream, float* out, long ldo, const float* r, const float* i, long ldg,
+                                   const float* u, long ldu, const float* y, long ldy, const void* lam, int w_dtype,
+                                   float decay, float* state, const int32_t* ent_slot, const int32_t* ent_row0,
+                                   const int32_t* ent_count, int E, int max_count, int C, void* ws, size_t ws_bytes);
 
 #ifdef __cplusplus
 }

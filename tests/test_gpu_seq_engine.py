@@ -147,3 +147,31 @@ def test_greedy_generation_through_the_scheduler():
     assert eng.state.used_pages() == 0 and not eng.state.live
     sampled = eng.generate(prompts[:2], max_new_tokens=4, sampling={"top_k": 5, "top_p": 0.9, "temperature": 0.8, "seed": 3})
     assert all(len(s) == 4 and all(0 <= x < cfg["vocab"] for x in s) for s in sampled)
+
+
+def test_decode_steps_replayed_as_graphs_equal_eager_steps(monkeypatch):
+    """bf16 decode steps of two requests: captured and replayed (several replays, eager work and synchronisation between
+    them) against the same steps launched eagerly, and a request that joins later (another graph)"""
+    cfg, t, rng = model("page", 7)
+    toks = [rng.integers(0, cfg["vocab"], n).tolist() for n in (90, 150, 40)]
+    def run(eng):
+        out = []
+        eng.step([("a", toks[0][:50], []), ("b", toks[1][:100], [])])
+        for i in range(25):
+            out.append(eng.step([("a", [toks[0][50 + i]], [0]), ("b", [toks[1][100 + i]], [0])]).cpu().numpy().copy())
+            if i == 10:
+                torch.cuda.synchronize()
+                eng.step([("c", toks[2][:30], [])])      # a prompt's portion between two replays
+        for i in range(10):
+            out.append(eng.step([("a", [toks[0][75 + i]], [0]), ("b", [toks[1][125 + i]], [0]), ("c", [toks[2][30 + i]], [0])]).cpu().numpy().copy())
+        return out
+    graphed = make_engine(cfg, t, torch.bfloat16)
+    assert graphed.use_graphs
+    got = run(graphed)
+    assert any(g["graph"] is not None for g in graphed._graphs.values())
+    monkeypatch.setenv("DIHIP_SEQ_GRAPH", "0")
+    eager = make_engine(cfg, t, torch.bfloat16)
+    assert not eager.use_graphs
+    want = run(eager)
+    for a, b in zip(got, want):
+        assert np.array_equal(a, b)

@@ -286,3 +286,44 @@ def test_latent_window_attn_on_the_matrix_cores(so, R, H, window, nsplit):
             shifted = attn_ref(qr, rows, pos, H, window + 1, 0.5, sink.float().numpy())
             if rel_err(shifted, want) > 0.05:
                 assert rel_err(got.cpu().numpy(), shifted) > 0.03
+
+
+def test_gated_recurrence_in_chunks_side_by_side(so):
+    """long portions cut into chunks that run in parallel: two portions of unequal length (one shorter than a chunk) that start
+    from states an earlier step left"""
+    rng = np.random.default_rng(12)
+    C, na, nb, pre = 70, 333, 40, 9
+    mk = lambda n: (rng.normal(0, 1, (n, C)).astype(np.float32), rng.normal(0, 1, (n, C)).astype(np.float32),
+                    rng.uniform(0, 1, (n, C)).astype(np.float32), rng.uniform(0, 1, (n, C)).astype(np.float32))
+    lam = bf(rng.normal(-2, 2, C))
+    seqs = [mk(pre + na), mk(pre + nb)]
+    want = [om.gated_recurrence(u.astype(np.float64), r, i, lam.double().numpy(), 8.0) * y for u, y, r, i in seqs]
+    state = torch.zeros(3, C, device="cuda")
+    cat = lambda k, lo, hi: dev(np.concatenate([seqs[0][k][lo[0]:hi[0]], seqs[1][k][lo[1]:hi[1]]]))
+    ts, to, es, er, ec = entries([(2, pre), (0, pre)], 3)
+    so.gated_recurrence(cat(2, (0, 0), (pre, pre)), cat(3, (0, 0), (pre, pre)), cat(0, (0, 0), (pre, pre)), cat(1, (0, 0), (pre, pre)), lam.cuda(),
+                        8.0, state, es, er, ec)
+    ts, to, es, er, ec = entries([(2, na), (0, nb)], 3)
+    lo, hi = (pre, pre), (pre + na, pre + nb)
+    got = so.gated_recurrence(cat(2, lo, hi), cat(3, lo, hi), cat(0, lo, hi), cat(1, lo, hi), lam.cuda(), 8.0, state, es, er, ec, max_count=na)
+    seq_state = state.clone()
+    assert rel_err(got[:na].cpu().numpy(), want[0][pre:]) < 5e-6 and rel_err(got[na:].cpu().numpy(), want[1][pre:]) < 5e-6
+    # the states it leaves are those of the row-by-row form
+    state2 = torch.zeros(3, C, device="cuda")
+    for (s, n), k in (((2, pre + na), 0), ((0, pre + nb), 1)):
+        ts, to, es, er, ec = entries([(s, n)], 3)
+        so.gated_recurrence(dev(seqs[k][2]), dev(seqs[k][3]), dev(seqs[k][0]), dev(seqs[k][1]), lam.cuda(), 8.0, state2, es, er, ec)
+    assert rel_err(seq_state.cpu().numpy(), state2.cpu().numpy()) < 5e-6 and float(seq_state[1].abs().max()) == 0
+
+
+@pytest.mark.parametrize("T", [1, 3, 4, 9, 40])
+def test_linear_f32_stream_mode(so, T):
+    """f32 products of the unrounded rows whichever kernel serves the row count (block-diagonal weights with bias and sigmoid)"""
+    rng = np.random.default_rng(T)
+    G, N, K = 6, 40, 40
+    x = rng.normal(0, 1, (T, 3 * K)).astype(np.float32)
+    w, b = bf(rng.normal(0, 0.2, (G, N, K))), bf(rng.normal(0, 0.3, (G, N)))
+    y = so.linear(dev(x), w.cuda(), b.cuda(), act="sigmoid", groups=G, x_groups=3, math=so.MATH_F32_STREAM)
+    want = np.concatenate([om.sigmoid(x[:, (g % 3) * K:(g % 3 + 1) * K].astype(np.float64) @ w[g].double().numpy().T + b[g].double().numpy())
+                           for g in range(G)], 1)
+    assert rel_err(y.cpu().numpy(), want) < 2e-6
