@@ -107,7 +107,8 @@ __device__ __forceinline__ u32x4_t load8_bf16(const void* p, size_t i, int kleft
 
 template <int XT, bool VEC>
 __global__ __launch_bounds__(256) void linear_mfma_kernel(LinArgs a) {
-  constexpr int LD = 40;  // bf16 elements per LDS row: 32 + 8 of padding (80 bytes: 16-byte aligned fragments)
+  constexpr int BK = 32, UPR = BK / 8, UN = 128 * UPR / 256;   // k per step (64 measured slower: fewer workgroups per CU), 16-byte units per tile row, units per thread
+  constexpr int LD = BK + 8;  // bf16 elements per LDS row: 8 of padding (144 bytes: 16-byte aligned fragments)
   __shared__ __attribute__((aligned(16))) uint16_t As[128 * LD];
   __shared__ __attribute__((aligned(16))) uint16_t Bs[128 * LD];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -121,35 +122,38 @@ __global__ __launch_bounds__(256) void linear_mfma_kernel(LinArgs a) {
   for (int i = 0; i < 4; ++i)
 #pragma unroll
     for (int j = 0; j < 4; ++j) acc[i][j] = z4;
-  u32x4_t ra[2], rb[2];
+  u32x4_t ra[UN], rb[UN];
   auto fetch = [&](int k0) {
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      const int u = tid + 256 * j, r = u >> 2, k = k0 + (u & 3) * 8;
+    for (int j = 0; j < UN; ++j) {
+      const int u = tid + 256 * j, r = u / UPR, k = k0 + (u % UPR) * 8;
       ra[j] = load8_bf16<XT, VEC>(a.x, (size_t)(m0 + r) * a.ldx + xoff + k, a.K - k, m0 + r < a.T);
       rb[j] = load8_bf16<DIHIP_BF16, VEC>(a.w, wbase + (size_t)(n0 + r) * a.K + k, a.K - k, n0 + r < a.N);
     }
   };
   fetch(0);
-  for (int k0 = 0; k0 < a.K; k0 += 32) {
+  for (int k0 = 0; k0 < a.K; k0 += BK) {
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      const int u = tid + 256 * j, r = u >> 2, kq = (u & 3) * 8;
+    for (int j = 0; j < UN; ++j) {
+      const int u = tid + 256 * j, r = u / UPR, kq = (u % UPR) * 8;
       *reinterpret_cast<u32x4_t*>(&As[r * LD + kq]) = ra[j];
       *reinterpret_cast<u32x4_t*>(&Bs[r * LD + kq]) = rb[j];
     }
     __syncthreads();
-    if (k0 + 32 < a.K) fetch(k0 + 32);
-    u32x4_t af[4], bf[4];
+    if (k0 + BK < a.K) fetch(k0 + BK);
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      af[i] = *reinterpret_cast<const u32x4_t*>(&As[(wm * 64 + i * 16 + (lane & 15)) * LD + (lane >> 4) * 8]);
-      bf[i] = *reinterpret_cast<const u32x4_t*>(&Bs[(wn * 64 + i * 16 + (lane & 15)) * LD + (lane >> 4) * 8]);
+    for (int ks = 0; ks < BK / 32; ++ks) {
+      u32x4_t af[4], bf[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        af[i] = *reinterpret_cast<const u32x4_t*>(&As[(wm * 64 + i * 16 + (lane & 15)) * LD + ks * 32 + (lane >> 4) * 8]);
+        bf[i] = *reinterpret_cast<const u32x4_t*>(&Bs[(wn * 64 + i * 16 + (lane & 15)) * LD + ks * 32 + (lane >> 4) * 8]);
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = mfma_bf16(af[i], bf[j], acc[i][j]);
     }
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-#pragma unroll
-      for (int j = 0; j < 4; ++j) acc[i][j] = mfma_bf16(af[i], bf[j], acc[i][j]);
     __syncthreads();
   }
   asm volatile("s_nop 15\n\ts_nop 7" ::: "memory");  // the matrix pipe's write-back before the results are read

@@ -131,10 +131,10 @@ def operator_table(size, prompt_len):
         for name, G, N, K, xg in (("attn q absorb", H, R, D, H), ("attn uv", H, V, R, H), ("rglru gates (f32)", 2 * B, C // B, C // B, B)):
             w = bf(G, N, K)
             y = torch.empty(T, G * N, device=dev)
-            mth = so.MATH_F32 if "gates" in name else so.MATH_BF16
+            mth = so.MATH_F32_STREAM if "gates" in name else so.MATH_BF16
             sec = _time(lambda: so.linear(x[:, :xg * K], w, out=y, math=mth, groups=G, x_groups=xg), 5)
             fl, by = 2.0 * T * G * N * K, 2.0 * G * N * K + 4.0 * T * (G * N + xg * K)
-            bound = max(fl / (VALU_F32 if mth == so.MATH_F32 else MFMA_BF16), by / HBM_BW)
+            bound = max(fl / (VALU_F32 if mth != so.MATH_BF16 else MFMA_BF16), by / HBM_BW)
             rows.append({"op": f"grouped linear {name} {G}x[{T}x{K}]x[{N}]", "us": round(sec * 1e6, 1), "tflops": round(fl / sec / 1e12, 2),
                          "of_bound": round(bound / sec, 3)})
         # attention over the cache: prompt rows at positions 0 .. T-1, or one row at position prompt_len - 1

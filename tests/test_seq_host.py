@@ -120,3 +120,22 @@ def test_registry_resolves_by_config():
         models.resolve({"architecture": "NoSuchModel"})
     with pytest.raises(KeyError):
         models.resolve({})
+
+
+def test_seq_library_exports_every_header_symbol():
+    """libdashinfer_hip_seq.so exports what include/dashinfer_hip_seq.h declares, and the ctypes table covers the header"""
+    import ctypes
+    import re
+    from dash_infer_amd import REPO_ROOT, seq_capi
+    assert os.path.exists(seq_capi.SEQ_LIB_PATH), "build with __graft_entry__.build()"
+    text = re.sub(r"/\*.*?\*/", "", open(os.path.join(REPO_ROOT, "include", "dashinfer_hip_seq.h")).read(), flags=re.S)
+    syms = sorted(set(re.findall(r"\b(dihip_[a-z0-9_]+)\s*\(", text)))
+    l = ctypes.CDLL(seq_capi.SEQ_LIB_PATH)
+    assert len(syms) >= 15 and not [s for s in syms if not hasattr(l, s)]
+    assert set(syms) == set(seq_capi._SIGS), set(syms) ^ set(seq_capi._SIGS)
+    lib = seq_capi.lib()
+    assert b"gfx950" in lib.dihip_seq_version()
+    assert lib.dihip_latent_window_attn_mc_supported(512, 64, seq_capi.BF16) == 1
+    assert lib.dihip_latent_window_attn_mc_supported(48, 64, seq_capi.BF16) == 0 and lib.dihip_latent_window_attn_mc_supported(64, 64, seq_capi.F32) == 0
+    assert lib.dihip_latent_window_attn_mc_workspace_bytes(4, 32, 512, 16) == 16 * 4 * 32 * 516 * 4
+    assert lib.dihip_gated_recurrence_chunked_workspace_bytes(2, 130, 100) == 2 * 3 * 2 * 100 * 4
