@@ -82,7 +82,8 @@ template <int WT>
 __global__ __launch_bounds__(256) void norm_residual_mix_kernel(float* x_out, const float* x_in, const float* __restrict__ m,
                                                                 long ldm, const void* __restrict__ gamma, float eps,
                                                                 float* stack_top, const float* __restrict__ stack, size_t stack_stride,
-                                                                const void* __restrict__ mix_w, int n_mix, float* __restrict__ x_mix, int K) {
+                                                                const void* __restrict__ mix_w, int n_mix, float* __restrict__ x_mix,
+                                                                uint16_t* __restrict__ next16, int K) {
   __shared__ float red[4];
   __shared__ float mw[256];
   const int t = blockIdx.x;
@@ -107,10 +108,13 @@ __global__ __launch_bounds__(256) void norm_residual_mix_kernel(float* x_out, co
       const int k = k0 + i * 256;
       if (k < K) {
         x_out[row + k] = xo[i];
+        float nx = xo[i];
         if (n_mix > 0) {
           stack_top[row + k] = xo[i];
-          x_mix[row + k] = __builtin_fmaf(mw[n_mix - 1], xo[i], mix[i]);
+          nx = __builtin_fmaf(mw[n_mix - 1], xo[i], mix[i]);
+          x_mix[row + k] = nx;
         }
+        if (next16) next16[row + k] = (uint16_t)f32_to_bf16_bits(nx);
       }
     }
   }
@@ -389,7 +393,8 @@ int dihip_norm_span_append(void* stream, void* const* spans, int span_stride, in
 }
 
 int dihip_norm_residual_mix(void* stream, float* x_out, const float* x_in, const float* m, long ldm, const void* gamma, int w_dtype,
-                            float eps, float* stack, size_t stack_stride, const void* mix_w, int n_mix, float* x_mix, int T, int K) {
+                            float eps, float* stack, size_t stack_stride, const void* mix_w, int n_mix, float* x_mix, void* next16, int T,
+                            int K) {
   DIHIP_REQUIRE(T >= 0 && K > 0 && x_out && x_in && m && gamma && ldm >= K && seq_dtype_ok(w_dtype), DIHIP_PARAM_ERROR,
                 "norm_residual_mix: bad argument");
   DIHIP_REQUIRE(n_mix == 0 || (stack && mix_w && x_mix && stack_stride >= (size_t)T * K && x_mix != x_out), DIHIP_PARAM_ERROR,
@@ -397,8 +402,8 @@ int dihip_norm_residual_mix(void* stream, float* x_out, const float* x_in, const
   if (T == 0) return DIHIP_SUCCESS;
   DIHIP_REQUIRE(n_mix <= 256, DIHIP_EXCEED_LIMIT_ERROR, "norm_residual_mix: more than 256 levels");
   float* top = n_mix > 0 ? stack + (size_t)(n_mix - 1) * stack_stride : nullptr;
-  if (w_dtype == DIHIP_F32) hipLaunchKernelGGL(norm_residual_mix_kernel<DIHIP_F32>, dim3(T), dim3(256), 0, reinterpret_cast<hipStream_t>(stream), x_out, x_in, m, ldm, gamma, eps, top, stack, stack_stride, mix_w, n_mix, x_mix, K);
-  else hipLaunchKernelGGL(norm_residual_mix_kernel<DIHIP_BF16>, dim3(T), dim3(256), 0, reinterpret_cast<hipStream_t>(stream), x_out, x_in, m, ldm, gamma, eps, top, stack, stack_stride, mix_w, n_mix, x_mix, K);
+  if (w_dtype == DIHIP_F32) hipLaunchKernelGGL(norm_residual_mix_kernel<DIHIP_F32>, dim3(T), dim3(256), 0, reinterpret_cast<hipStream_t>(stream), x_out, x_in, m, ldm, gamma, eps, top, stack, stack_stride, mix_w, n_mix, x_mix, (uint16_t*)next16, K);
+  else hipLaunchKernelGGL(norm_residual_mix_kernel<DIHIP_BF16>, dim3(T), dim3(256), 0, reinterpret_cast<hipStream_t>(stream), x_out, x_in, m, ldm, gamma, eps, top, stack, stack_stride, mix_w, n_mix, x_mix, (uint16_t*)next16, K);
   return launch_status();
 }
 

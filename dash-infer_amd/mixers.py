@@ -26,6 +26,11 @@ class StepContext:
         self.max_count, self.max_pos = T, 0     # host numbers: the largest portion and the last position of the step
         self.taps = None    # layer index -> [T, .] intermediate (diagnostics; None: off)
 
+    def act_buffer(self, n, dtype=None):
+        """[T, n] for an activation that only a product reads: bf16 under bf16 products (the product would round it anyway), else f32"""
+        dt = dtype or (torch.bfloat16 if self.math == so.MATH_BF16 else torch.float32)
+        return torch.empty(self.T, n, dtype=dt, device=self.ids.device)
+
 
 class LatentWindowAttention:
     def __init__(self, key, heads, dim, vdim, kv_rank, q_rank, window, scale, w, state, cache_dtype, kv_from_key=None):
@@ -52,10 +57,11 @@ class LatentWindowAttention:
             assert self.table.row_elems == kv_rank, "a shared latent cache must have this layer's rank"
         self.mc = so.latent_attn_mc_supported(self.table) and (heads * kv_rank) % 4 == 0
 
-    def __call__(self, ctx, h):
-        a = so.linear(h, self.w_in, act="sigmoid", act_cols=(self.g_lo, self.n_in), math=ctx.math)
-        cq = so.rmsnorm(a[:, : self.Q], self.dq_norm, ctx.eps)
-        q = so.linear(cq, self.uq, math=ctx.math)
+    def __call__(self, ctx, h, h16=None):
+        """h16: the bf16 copy of h where the producer made one (bf16 products read it: the same bits at half the traffic)"""
+        a = so.linear(h16 if h16 is not None else h, self.w_in, act="sigmoid", act_cols=(self.g_lo, self.n_in), math=ctx.math)
+        cq = so.rmsnorm(a[:, : self.Q], self.dq_norm, ctx.eps, out=ctx.act_buffer(self.Q))
+        q = so.linear(cq, self.uq, math=ctx.math, out=ctx.act_buffer(self.H * self.D))
         if self.owns_cache:
             so.norm_span_append(self.table, a[:, self.c_lo: self.g_lo], self.dkv_norm, ctx.eps, ctx.tok_slot, ctx.tok_pos)
         ql = so.linear(q, self.uk_t, groups=self.H, math=ctx.math)
@@ -64,7 +70,7 @@ class LatentWindowAttention:
                                           ctx.max_pos, self.H, self.window, self.scale)
         else:
             ol = so.latent_window_attn(ql, self.table, self.sink, ctx.tok_slot, ctx.tok_pos, self.H, self.window, self.scale, math=ctx.math)
-        og = so.linear(ol, self.uv, groups=self.H, mul=a[:, self.g_lo:], math=ctx.math)
+        og = so.linear(ol, self.uv, groups=self.H, mul=a[:, self.g_lo:], math=ctx.math, out=ctx.act_buffer(self.H * self.V))
         return so.linear(og, self.o, math=ctx.math)
 
 
@@ -83,9 +89,9 @@ class GatedLinearRecurrence:
         self.S = state.add_state(key + ".S", (width,))
         self.tail = state.add_state(key + ".tail", (taps - 1, width)) if taps > 1 else None
 
-    def __call__(self, ctx, h):
+    def __call__(self, ctx, h, h16=None):
         C = self.C
-        a = so.linear(h, self.w_in, self.b_in, act="gelu_tanh", act_cols=(0, C), math=ctx.math)     # [y | x]
+        a = so.linear(h16 if h16 is not None else h, self.w_in, self.b_in, act="gelu_tanh", act_cols=(0, C), math=ctx.math)     # [y | x]
         y, x = a[:, :C], a[:, C:]
         u = so.causal_conv_state(x, self.conv, self.conv_b, self.tail, ctx.tok_slot, ctx.tok_off)
         if self.tail is not None:
@@ -101,5 +107,6 @@ class DenseMlp:
     def __init__(self, up, down, act):
         self.up, self.down, self.act = up.contiguous(), down.contiguous(), act
 
-    def __call__(self, ctx, h):
-        return so.linear(so.linear(h, self.up, act=self.act, math=ctx.math), self.down, math=ctx.math)
+    def __call__(self, ctx, h, h16=None):
+        act = so.linear(h16 if h16 is not None else h, self.up, act=self.act, math=ctx.math, out=ctx.act_buffer(self.up.shape[0]))
+        return so.linear(act, self.down, math=ctx.math)

@@ -90,23 +90,26 @@ class Modanex:
         dev = self.embed.device
         stack = torch.empty(L + 1, T, W, dtype=torch.float32, device=dev)
         so.embed_sum(ctx.ids, self.embed, ctx.rows2, self.bigram, out=stack[0])
-        cur = stack[0]
+        cur, cur16 = stack[0], None
+        bf = self.math == so.MATH_BF16      # bf16 copies of what the products read, written by the kernel that makes the f32 rows
         xr = torch.empty(T, W, dtype=torch.float32, device=dev)
+        xr16 = torch.empty(T, W, dtype=torch.bfloat16, device=dev) if bf else None
         mixed = [torch.empty(T, W, dtype=torch.float32, device=dev) for _ in range(2)]
+        mixed16 = [torch.empty(T, W, dtype=torch.bfloat16, device=dev) if bf else None for _ in range(2)]
         for i, (mixer, norm1, mlp, norm2, dwa) in enumerate(self.layers):
             n_mix = i + 2 if dwa is not None else 0
-            nxt = mixed[i & 1] if n_mix else xr
-            mo = mixer(ctx, cur)
+            nxt, nxt16 = (mixed[i & 1], mixed16[i & 1]) if n_mix else (xr, xr16)
+            mo = mixer(ctx, cur, cur16)
             if mlp is None:
-                so.norm_residual_mix(cur, mo, norm1, ctx.eps, xr, stack, dwa, n_mix, nxt if n_mix else None)
+                so.norm_residual_mix(cur, mo, norm1, ctx.eps, xr, stack, dwa, n_mix, nxt if n_mix else None, next16=nxt16)
             else:
-                so.norm_residual_mix(cur, mo, norm1, ctx.eps, xr)
-                f = mlp(ctx, xr)
-                so.norm_residual_mix(xr, f, norm2, ctx.eps, xr, stack, dwa, n_mix, nxt if n_mix else None)
+                so.norm_residual_mix(cur, mo, norm1, ctx.eps, xr, next16=xr16)
+                f = mlp(ctx, xr, xr16)
+                so.norm_residual_mix(xr, f, norm2, ctx.eps, xr, stack, dwa, n_mix, nxt if n_mix else None, next16=nxt16)
             if not n_mix:      # no depth average: the layer's result goes on as it is
-                nxt = xr
                 xr = torch.empty(T, W, dtype=torch.float32, device=dev)
-            cur = nxt
+                xr16 = torch.empty(T, W, dtype=torch.bfloat16, device=dev) if bf else None
+            cur, cur16 = nxt, nxt16
             if ctx.taps is not None:
                 ctx.taps[i] = cur.clone()
         return cur

@@ -24,7 +24,7 @@ _SIGS = {
     "dihip_embed_sum": (i32, [vp, vp, vp, vp, vp, vp, i32, i32, i32]),
     "dihip_rmsnorm_strided": (i32, [vp, vp, i32, lng, vp, lng, vp, vp, i32, f32, i32, i32]),
     "dihip_norm_span_append": (i32, [vp, vp, i32, i32, i32, vp, lng, vp, i32, f32, vp, vp, i32, i32]),
-    "dihip_norm_residual_mix": (i32, [vp, vp, vp, vp, lng, vp, i32, f32, vp, sz, vp, i32, vp, i32, i32]),
+    "dihip_norm_residual_mix": (i32, [vp, vp, vp, vp, lng, vp, i32, f32, vp, sz, vp, i32, vp, vp, i32, i32]),
     "dihip_latent_window_attn": (i32, [vp, vp, lng, vp, lng, vp, i32, i32, i32, vp, i32, vp, vp, i32, i32, i32, i32, f32, i32]),
     "dihip_latent_window_attn_mc_supported": (i32, [i32, i32, i32]),
     "dihip_latent_window_attn_mc_workspace_bytes": (sz, [i32, i32, i32, i32]),

@@ -79,13 +79,15 @@ def norm_span_append(table, x, gamma, eps, tok_slot, tok_pos):
                                        ptr(gamma), dt(gamma), float(eps), ptr(tok_slot), ptr(tok_pos), T, K), "dihip_norm_span_append")
 
 
-def norm_residual_mix(x_in, m, gamma, eps, x_out, stack=None, mix_w=None, n_mix=0, x_mix=None):
+def norm_residual_mix(x_in, m, gamma, eps, x_out, stack=None, mix_w=None, n_mix=0, x_mix=None, next16=None):
+    """next16: optional bf16 [T, K] copy of what the next product reads (x_mix where n_mix > 0, else x_out)"""
     T, K = x_in.shape
     assert x_in.is_contiguous() and x_out.is_contiguous() and m.shape == (T, K)
+    assert next16 is None or (next16.dtype == torch.bfloat16 and next16.is_contiguous() and next16.shape == (T, K))
     if n_mix:
         assert stack.is_contiguous() and stack.shape[0] >= n_mix and x_mix.is_contiguous() and mix_w.shape[0] >= n_mix
     check(lib().dihip_norm_residual_mix(stream(), ptr(x_out), ptr(x_in), ptr(m), _rows(m), ptr(gamma), dt(gamma), float(eps),
-                                        ptr(stack), stack.stride(0) if n_mix else 0, ptr(mix_w), n_mix, ptr(x_mix), T, K),
+                                        ptr(stack), stack.stride(0) if n_mix else 0, ptr(mix_w), n_mix, ptr(x_mix), ptr(next16), T, K),
           "dihip_norm_residual_mix")
     return x_out
 

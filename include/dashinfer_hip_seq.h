@@ -55,10 +55,12 @@ int dihip_norm_span_append(void* stream, void* const* spans, int span_stride, in
 /* The residual step with the norm on the sublayer's OUTPUT and the depth-weighted stream:
  *   x_out[t] = x_in[t] + rmsnorm(m[t]; gamma, eps)
  *   n_mix > 0:  stack[n_mix - 1][t] = x_out[t];  x_mix[t] = sum_{j < n_mix} mix_w[j] * stack[j][t]
- * stack: [.][stack_stride] f32 (stack_stride >= T * K elements per level); x_out may alias x_in. */
+ * stack: [.][stack_stride] f32 (stack_stride >= T * K elements per level); x_out may alias x_in.
+ * next16 (may be NULL): [T, K] bf16 copy of what the next product reads (x_mix where n_mix > 0, else x_out): the product
+ * rounds its operand to bf16 anyway, so reading the copy changes no bit and halves its operand traffic. */
 int dihip_norm_residual_mix(void* stream, float* x_out, const float* x_in, const float* m, long ldm,
                             const void* gamma, int w_dtype, float eps, float* stack, size_t stack_stride,
-                            const void* mix_w, int n_mix, float* x_mix, int T, int K);
+                            const void* mix_w, int n_mix, float* x_mix, void* next16, int T, int K);
 
 /* Windowed attention of every row over its sequence's cached latent rows, all heads sharing the cache:
  *   s_j = scale * q[t, h, :] . c_j   for  0 <= tok_pos[t] - j < window  (window <= 0: every j <= tok_pos[t]),
