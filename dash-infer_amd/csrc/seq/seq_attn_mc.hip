@@ -81,30 +81,32 @@ __global__ __launch_bounds__(256) void latent_attn_mc_kernel(McArgs a) {
     tabs[i] = (sp * a.span_len <= p_hi) ? (const char*)gtab[sp] : nullptr;
   }
   __syncthreads();
+  // a thread's 16-byte units of a tile: (key inside the tile, column) fixed for the whole walk -- the divisions are done once.
+  // A tile of 32 keys lies inside one span (span_len % 32 == 0): its span and offset are wave-uniform.
   const int upr = R >> 3;  // 16-byte units per cached row
+  int goff[UN], loff[UN];
+#pragma unroll
+  for (int j = 0; j < UN; ++j) {
+    const int u = tid + 256 * j, kin = u / upr, c8 = u - kin * upr;
+    goff[j] = kin < 32 ? (kin * R + c8 * 8) * 2 : -1;
+    loff[j] = kin * pitchb + c8 * 16;
+  }
   u32x4_t pre[UN];
   auto fetch = [&](int tile) {
+    const int key0 = tile * 32, sp = key0 / a.span_len;
+    const char* sb = (sp - span_lo < 128 ? tabs[sp - span_lo] : (const char*)gtab[sp]) + (size_t)(key0 - sp * a.span_len) * R * 2;
 #pragma unroll
     for (int j = 0; j < UN; ++j) {
-      const int u = tid + 256 * j, kin = u / upr, c8 = u - kin * upr;
       pre[j] = u32x4_t{0u, 0u, 0u, 0u};
-      if (kin < 32) {
-        const int key = tile * 32 + kin;
-        const int sp = key / a.span_len;
-        const char* sb = sp - span_lo < 128 ? tabs[sp - span_lo] : (const char*)gtab[sp];
-        const char* src = sb + ((size_t)(key - sp * a.span_len) * R + c8 * 8) * 2;
-        pre[j] = gload<u32x4_t>(src);
-      }
+      if (goff[j] >= 0) pre[j] = gload<u32x4_t>(sb + goff[j]);
     }
   };
   if (PREFETCH && my_lo <= my_hi) fetch(my_lo);
   for (int tile = my_lo; tile <= my_hi; ++tile) {
     if (!PREFETCH) fetch(tile);
 #pragma unroll
-    for (int j = 0; j < UN; ++j) {
-      const int u = tid + 256 * j, kin = u / upr, c8 = u - kin * upr;
-      if (kin < 32) *reinterpret_cast<u32x4_t*>(smem + kin * pitchb + c8 * 16) = pre[j];
-    }
+    for (int j = 0; j < UN; ++j)
+      if (goff[j] >= 0) *reinterpret_cast<u32x4_t*>(smem + loff[j]) = pre[j];
     __syncthreads();
     if (PREFETCH && tile + 1 <= my_hi) fetch(tile + 1);
     f32x4_t sacc[2] = {z4, z4};
@@ -130,14 +132,14 @@ __global__ __launch_bounds__(256) void latent_attn_mc_kernel(McArgs a) {
       }
     mx = rows_max(mx);
     const float mn = fmaxf(m, mx);
-    const float corr = expf(m - mn);
+    const float corr = __expf(m - mn);
     m = mn;
     float psum = 0.f, ev[2][4];
 #pragma unroll
     for (int nt = 0; nt < 2; ++nt)
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
-        ev[nt][r] = expf(sv[nt][r] - mn);
+        ev[nt][r] = __expf(sv[nt][r] - mn);
         psum += ev[nt][r];
       }
     l = l * corr + rows_sum(psum);
