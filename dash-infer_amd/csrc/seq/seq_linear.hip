@@ -108,7 +108,7 @@ __device__ __forceinline__ u32x4_t load8_bf16(const void* p, size_t i, int kleft
 template <int XT, bool VEC>
 __global__ __launch_bounds__(256) void linear_mfma_kernel(LinArgs a) {
   constexpr int BK = 32, UPR = BK / 8, UN = 128 * UPR / 256;   // k per step (64 measured slower: fewer workgroups per CU), 16-byte units per tile row, units per thread
-  constexpr int LD = BK + 8;  // bf16 elements per LDS row: 8 of padding (144 bytes: 16-byte aligned fragments)
+  constexpr int LD = BK + 8;  // bf16 elements per LDS row: 8 of padding (80 bytes: 16-byte aligned fragments)
   __shared__ __attribute__((aligned(16))) uint16_t As[128 * LD];
   __shared__ __attribute__((aligned(16))) uint16_t Bs[128 * LD];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
