@@ -129,10 +129,17 @@ class SeqEngine:
         logits = self.model.logits(ctx, self.model.forward(ctx), ctx.want_rows)
         if (E, bucket) in self._graphs:
             torch.cuda.synchronize()
-            graph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(graph):      # records the same launches; nothing runs, the state is not touched
-                g["logits"] = self.model.logits(ctx, self.model.forward(ctx), ctx.want_rows)
-            g["graph"] = graph
+            try:
+                graph = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(graph):      # records the same launches; nothing runs, the state is not touched
+                    g["logits"] = self.model.logits(ctx, self.model.forward(ctx), ctx.want_rows)
+                g["graph"] = graph
+            except Exception as e:  # noqa: BLE001  a capture that fails costs speed only: this step has run, later ones launch eagerly
+                import sys
+                print(f"sequence engine: hipGraph capture failed ({type(e).__name__}: {e}); decode steps launch eagerly", file=sys.stderr)
+                self.use_graphs = False
+                self._graphs.clear()
+                torch.cuda.synchronize()
         return logits
 
     def release(self, rid):
