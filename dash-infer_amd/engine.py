@@ -120,8 +120,12 @@ class SeqEngine:
                  "meta": torch.empty(host.numel(), dtype=torch.int32, device=self.device), "graph": None}
             if len(self._graphs) < 64:
                 self._graphs[(E, bucket)] = g
+        if "copied" in g:
+            g["copied"].synchronize()      # the staging block is free again once the step before has read it
         g["host"].copy_(host)
         g["meta"].copy_(g["host"], non_blocking=True)
+        g["copied"] = torch.cuda.Event()
+        g["copied"].record()
         if g["graph"] is not None:
             g["graph"].replay()
             return g["logits"]
