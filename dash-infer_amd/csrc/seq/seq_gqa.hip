@@ -1,0 +1,513 @@
+// seq_gqa.hip -- grouped-query attention over paged key and value caches for the sequence engine:
+//   qkv_prep_append   per token: unit-RMS norm of every query / key head (optional), rotary positions (paired or half-split
+//                     layout, a frequency table and a magnitude from the host), mixing of the values with another layer's,
+//                     queries written back in place, keys and values appended to their pages
+//   gqa_attn_kernel   one workgroup per row, every product and sum in f32 (any cache type)
+//   gqa_attn_mc_kernel + merge   bf16 caches on the matrix cores, the key walk split for few rows (decoding)
+// Options of the softmax: a sink logit per head or the constant 0 (one more term in the denominator, no value), a tanh cap on
+// the scores, a multiplier per (row, head) on the output (the output gate).
+#include "seq_common.h"
+
+namespace dihip {
+namespace {
+
+// ------------------------------------------------------------------------------------------------ prep + append
+struct PrepArgs {
+  float* qkv; long ld; int q_off, k_off, v_off;
+  int H, G, D, DV;
+  const void* qnorm; const void* knorm; int wdt; float eps;
+  const float* freq; int rot_dims, layout; float mag;
+  float lam; const float* vfirst_in; float* vfirst_out; long ldvf;
+  void* const* kspans; void* const* vspans; int span_stride, span_len, cdt;
+  const int32_t* tok_slot; const int32_t* tok_pos;
+};
+
+__global__ __launch_bounds__(256) void qkv_prep_append_kernel(PrepArgs a) {
+  __shared__ float hs[4][256];
+  const int t = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int pos = a.tok_pos[t];
+  const size_t sp = (size_t)a.tok_slot[t] * a.span_stride + pos / a.span_len;
+  const size_t in_span = (size_t)(pos % a.span_len);
+  float* row = a.qkv + (size_t)t * a.ld;
+  const int D = a.D, half = a.rot_dims >> 1;
+  for (int h0 = 0; h0 < a.H + a.G; h0 += 4) {      // query heads, then key heads: the same trip count in every wave
+    const int hh = h0 + wave;
+    const bool live = hh < a.H + a.G, is_q = hh < a.H;
+    float* src = row + (is_q ? a.q_off + hh * D : a.k_off + (hh - a.H) * D);
+    const void* gamma = is_q ? a.qnorm : a.knorm;
+    float v[4], ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int d = lane + 64 * i;
+      v[i] = live && d < D ? src[d] : 0.f;
+      ss = __builtin_fmaf(v[i], v[i], ss);
+    }
+    if (gamma) {
+      const float inv = 1.f / sqrtf(wave_sum(ss) / (float)D + a.eps);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int d = lane + 64 * i;
+        if (d < D) v[i] = v[i] * inv * ld_any(gamma, d, a.wdt);
+      }
+    }
+    __syncthreads();   // hs of the head before is no longer read
+#pragma unroll
+    for (int i = 0; i < 4; ++i) hs[wave][lane + 64 * i] = v[i];
+    __syncthreads();
+    if (live) {
+      void* kdst = is_q ? nullptr : a.kspans[sp];
+      const size_t kbase = (in_span * a.G + (size_t)(is_q ? 0 : hh - a.H)) * D;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int d = lane + 64 * i;
+        if (d >= D) continue;
+        float y = v[i];
+        if (d < a.rot_dims) {
+          int pair, other;
+          bool first;
+          if (a.layout == 0) { pair = d >> 1; first = (d & 1) == 0; other = d ^ 1; }
+          else { first = d < half; pair = first ? d : d - half; other = first ? d + half : d - half; }
+          float sn, cs;
+          rope_sincos((uint32_t)pos, a.freq[pair], &sn, &cs);
+          sn *= a.mag; cs *= a.mag;
+          const float o = hs[wave][other];
+          y = first ? v[i] * cs - o * sn : v[i] * cs + o * sn;
+        }
+        if (is_q) src[d] = y;
+        else st_any(kdst, kbase + d, a.cdt, y);
+      }
+    }
+  }
+  void* vdst = a.vspans[sp];
+  const int nv = a.G * a.DV;
+  for (int e = threadIdx.x; e < nv; e += 256) {
+    float v = row[a.v_off + e];
+    if (a.vfirst_in) v = (1.f - a.lam) * v + a.lam * a.vfirst_in[(size_t)t * a.ldvf + e];
+    if (a.vfirst_out) a.vfirst_out[(size_t)t * a.ldvf + e] = v;
+    st_any(vdst, in_span * nv + e, a.cdt, v);
+  }
+}
+
+// ------------------------------------------------------------------------------------------------ f32 row kernel
+struct GqaArgs {
+  float* out; long ldo;
+  const float* q; long ldq;
+  void* const* kspans; void* const* vspans; int span_stride, span_len;
+  const void* sink; int wdt, sink_mode;   // 0: none, 1: sink[h], 2: the constant 0
+  float softcap;                          // <= 0: none
+  const float* gate; long ldg;            // [T, H] multiplier (NULL: none)
+  const int32_t* tok_slot; const int32_t* tok_pos; const int32_t* ent_slot; const int32_t* ent_row0; const int32_t* ent_count;
+  int H, G, D, DV; float scale;
+  float* ws; int rows_total;
+};
+
+__device__ __forceinline__ float cap_score(float s, float cap) { return cap > 0.f ? cap * tanhf(s / cap) : s; }
+
+// One workgroup per row, its 4 waves take the heads in turn; a wave walks the keys 64 at a time: lane j scores key j (d
+// ascending), the chunk joins the running softmax, then the lanes turn to the value elements and add the weighted rows.
+template <int CT, int RV>
+__global__ __launch_bounds__(256) void gqa_attn_kernel(GqaArgs a) {
+  __shared__ float qs[4][256];
+  __shared__ float ps[4][64];
+  const int t = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int pos = a.tok_pos[t], H = a.H, G = a.G, D = a.D, DV = a.DV, hpg = H / G;
+  void* const* ktab = a.kspans + (size_t)a.tok_slot[t] * a.span_stride;
+  void* const* vtab = a.vspans + (size_t)a.tok_slot[t] * a.span_stride;
+  constexpr size_t ES = CT == DIHIP_F32 ? 4 : 2;
+  for (int h0 = 0; h0 < H; h0 += 4) {
+    const int h = h0 + wave;
+    const bool live = h < H;
+    const int g = (live ? h : 0) / hpg;
+    __syncthreads();
+    if (live)
+      for (int d = lane; d < D; d += 64) qs[wave][d] = a.q[(size_t)t * a.ldq + (size_t)h * D + d];
+    __syncthreads();
+    float mx = -INFINITY, den = 0.f;
+    if (a.sink_mode == 1) { mx = ld_any(a.sink, live ? h : 0, a.wdt); den = 1.f; }
+    else if (a.sink_mode == 2) { mx = 0.f; den = 1.f; }
+    float acc[RV];
+#pragma unroll
+    for (int v = 0; v < RV; ++v) acc[v] = 0.f;
+    for (int j0 = 0; j0 <= pos; j0 += 64) {
+      const int j = j0 + lane;
+      const bool valid = live && j <= pos;
+      float s = -INFINITY;
+      if (valid) {
+        const char* kr = (const char*)ktab[j / a.span_len] + ((size_t)(j % a.span_len) * G + g) * D * ES;
+        float d = 0.f;
+        for (int r = 0; r < D; ++r) d = __builtin_fmaf(qs[wave][r], load_ft<CT>(kr, r), d);
+        s = cap_score(d * a.scale, a.softcap);
+      }
+      const float mnew = fmaxf(mx, wave_max(s));
+      const float corr = mx == -INFINITY ? 0.f : expf(mx - mnew);
+      const float p = valid ? expf(s - mnew) : 0.f;
+      den = den * corr + wave_sum(p);
+#pragma unroll
+      for (int v = 0; v < RV; ++v) acc[v] *= corr;
+      mx = mnew;
+      ps[wave][lane] = p;
+      __syncthreads();
+      if (live) {
+        const int cnt = min(64, pos - j0 + 1);
+        for (int jj = 0; jj < cnt; ++jj) {
+          const int jk = j0 + jj;
+          const char* vr = (const char*)vtab[jk / a.span_len] + ((size_t)(jk % a.span_len) * G + g) * DV * ES;
+          const float pj = ps[wave][jj];
+#pragma unroll
+          for (int v = 0; v < RV; ++v) {
+            const int r = v * 64 + lane;
+            if (r < DV) acc[v] = __builtin_fmaf(pj, load_ft<CT>(vr, r), acc[v]);
+          }
+        }
+      }
+      __syncthreads();
+    }
+    if (live) {
+      const float gt = a.gate ? a.gate[(size_t)t * a.ldg + h] : 1.f;
+#pragma unroll
+      for (int v = 0; v < RV; ++v) {
+        const int r = v * 64 + lane;
+        if (r < DV) a.out[(size_t)t * a.ldo + (size_t)h * DV + r] = acc[v] / den * gt;
+      }
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------------------------ matrix-core kernel
+// A workgroup owns 64 consecutive (row, query head) pairs of ONE portion and ONE key/value head -- 16 per wave -- and walks
+// the 32-key tiles those pairs can see.  Per tile: S^T = K . Q^T (the tile's key rows as they lie in LDS against the wave's
+// query fragments, held in registers for the whole walk), cap + mask + running softmax on the accumulator lanes, then
+// O^T += V^T . P^T with P straight from those lanes and V^T read from the value tile through the transposing LDS read.  The
+// next tile's rows are in flight meanwhile.  Head sizes that are no multiple of the tile's granule are padded with zero
+// columns in LDS.  The key walk can be split over gridDim.z workgroups; the partial records are merged by a second launch.
+__device__ __forceinline__ f32x4_t mfma_bf16g(const u32x4_t& a, const u32x4_t& b, const f32x4_t& c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
+}
+__device__ __forceinline__ float fast_tanh(float x) { return 1.f - 2.f / (1.f + __expf(2.f * x)); }
+
+template <int DMAX, int VMAX>
+__global__ __launch_bounds__(256) void gqa_attn_mc_kernel(GqaArgs a) {
+  constexpr int KS = DMAX / 32, DT = VMAX / 16, UNK = DMAX / 64, UNV = VMAX / 64;
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  const int G = a.G, H = a.H, D = a.D, DV = a.DV, hpg = H / G;
+  const int e = blockIdx.y / G, g = blockIdx.y - e * G, split = blockIdx.z, nsplit = gridDim.z;
+  const int cnt = a.ent_count[e], row0 = a.ent_row0[e];
+  const int nrows = cnt * hpg, r0 = blockIdx.x * 64;
+  if (r0 >= nrows) return;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, ni = lane & 15, kb = lane >> 4;
+  const int Dp = (D + 31) & ~31, Vp = (DV + 15) & ~15;
+  const int pitchk = (Dp + 8) * 2, pitchv = (Vp + 8) * 2;
+  unsigned char* ksm = smem;
+  unsigned char* vsm = smem + 32 * pitchk;
+  const int pos0 = a.tok_pos[row0];
+  const int myrow = r0 + wave * 16 + ni;
+  const bool row_ok = myrow < nrows;
+  const int rr = row_ok ? myrow : nrows - 1;
+  const int tq = rr / hpg, h = g * hpg + (rr - tq * hpg), p = pos0 + tq;
+  const int p_hi = pos0 + min(r0 + 63, nrows - 1) / hpg;
+  const int tile_hi = p_hi >> 5;
+  const int per = (tile_hi + nsplit) / nsplit;
+  const int my_lo = split * per, my_hi = min(tile_hi, my_lo + per - 1);
+
+  u32x4_t qf[KS];
+  {
+    const float* qrow = a.q + (size_t)(row0 + tq) * a.ldq + (size_t)h * D;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      qf[ks] = u32x4_t{0u, 0u, 0u, 0u};
+      const int d0 = ks * 32 + kb * 8;
+      if (d0 < D) {   // D % 8 == 0: a unit of 8 is inside or outside
+        const f32x4_t lo = *reinterpret_cast<const f32x4_t*>(qrow + d0);
+        const f32x4_t hi = *reinterpret_cast<const f32x4_t*>(qrow + d0 + 4);
+        qf[ks] = u32x4_t{pack_bf16x2(lo[0], lo[1]), pack_bf16x2(lo[2], lo[3]), pack_bf16x2(hi[0], hi[1]), pack_bf16x2(hi[2], hi[3])};
+      }
+    }
+  }
+  const bool with_sink = a.sink_mode != 0 && split == 0;
+  float m = with_sink ? (a.sink_mode == 1 ? ld_any(a.sink, h, a.wdt) : 0.f) : -1e30f;
+  float l = with_sink ? 1.f : 0.f;
+  const f32x4_t z4 = {0.f, 0.f, 0.f, 0.f};
+  f32x4_t oacc[DT];
+#pragma unroll
+  for (int t = 0; t < DT; ++t) oacc[t] = z4;
+
+  // zero the padding columns once: the tiles' stores never touch them
+  for (int i = tid; i < 32 * (Dp - D + 8); i += 256) {
+    const int kin = i / (Dp - D + 8), c = D + i % (Dp - D + 8);
+    reinterpret_cast<uint16_t*>(ksm + kin * pitchk)[c] = 0;
+  }
+  for (int i = tid; i < 32 * (Vp - DV + 8); i += 256) {
+    const int kin = i / (Vp - DV + 8), c = DV + i % (Vp - DV + 8);
+    reinterpret_cast<uint16_t*>(vsm + kin * pitchv)[c] = 0;
+  }
+  __shared__ const char* ktabs[128];
+  __shared__ const char* vtabs[128];
+  void* const* gk = a.kspans + (size_t)a.ent_slot[e] * a.span_stride;
+  void* const* gv = a.vspans + (size_t)a.ent_slot[e] * a.span_stride;
+  const int span_lo = (my_lo * 32) / a.span_len;
+  for (int i = tid; i < 128; i += 256) {
+    const int sp = span_lo + i;
+    const bool in = sp * a.span_len <= p_hi;
+    ktabs[i] = in ? (const char*)gk[sp] : nullptr;
+    vtabs[i] = in ? (const char*)gv[sp] : nullptr;
+  }
+  __syncthreads();
+  const int uprk = D >> 3, uprv = DV >> 3;
+  int gok[UNK], lok[UNK], gov[UNV], lov[UNV];
+#pragma unroll
+  for (int j = 0; j < UNK; ++j) {
+    const int u = tid + 256 * j, kin = u / uprk, c8 = u - kin * uprk;
+    gok[j] = kin < 32 ? ((kin * G + g) * D + c8 * 8) * 2 : -1;
+    lok[j] = kin * pitchk + c8 * 16;
+  }
+#pragma unroll
+  for (int j = 0; j < UNV; ++j) {
+    const int u = tid + 256 * j, kin = u / uprv, c8 = u - kin * uprv;
+    gov[j] = kin < 32 ? ((kin * G + g) * DV + c8 * 8) * 2 : -1;
+    lov[j] = kin * pitchv + c8 * 16;
+  }
+  u32x4_t prek[UNK], prev[UNV];
+  auto fetch = [&](int tile) {
+    const int key0 = tile * 32, sp = key0 / a.span_len, in = key0 - sp * a.span_len;
+    const bool near = sp - span_lo < 128;
+    const char* kbp = (near ? ktabs[sp - span_lo] : (const char*)gk[sp]) + (size_t)in * G * D * 2;
+    const char* vbp = (near ? vtabs[sp - span_lo] : (const char*)gv[sp]) + (size_t)in * G * DV * 2;
+#pragma unroll
+    for (int j = 0; j < UNK; ++j) {
+      prek[j] = u32x4_t{0u, 0u, 0u, 0u};
+      if (gok[j] >= 0) prek[j] = gload<u32x4_t>(kbp + gok[j]);
+    }
+#pragma unroll
+    for (int j = 0; j < UNV; ++j) {
+      prev[j] = u32x4_t{0u, 0u, 0u, 0u};
+      if (gov[j] >= 0) prev[j] = gload<u32x4_t>(vbp + gov[j]);
+    }
+  };
+  if (my_lo <= my_hi) fetch(my_lo);
+  for (int tile = my_lo; tile <= my_hi; ++tile) {
+#pragma unroll
+    for (int j = 0; j < UNK; ++j)
+      if (gok[j] >= 0) *reinterpret_cast<u32x4_t*>(ksm + lok[j]) = prek[j];
+#pragma unroll
+    for (int j = 0; j < UNV; ++j)
+      if (gov[j] >= 0) *reinterpret_cast<u32x4_t*>(vsm + lov[j]) = prev[j];
+    __syncthreads();
+    if (tile + 1 <= my_hi) fetch(tile + 1);
+    f32x4_t sacc[2] = {z4, z4};
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      if (ks * 32 < D) {
+#pragma unroll
+        for (int nt = 0; nt < 2; ++nt) {
+          const u32x4_t kf = *reinterpret_cast<const u32x4_t*>(ksm + (nt * 16 + ni) * pitchk + (ks * 32 + kb * 8) * 2);
+          sacc[nt] = mfma_bf16g(kf, qf[ks], sacc[nt]);
+        }
+      }
+    }
+    float sv[2][4], mx = -INFINITY;
+#pragma unroll
+    for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int key = tile * 32 + nt * 16 + kb * 4 + r;
+        float s = sacc[nt][r] * a.scale;
+        if (a.softcap > 0.f) s = a.softcap * fast_tanh(s / a.softcap);
+        sv[nt][r] = key <= p ? s : -INFINITY;
+        mx = fmaxf(mx, sv[nt][r]);
+      }
+    mx = rows_max(mx);
+    const float mn = fmaxf(m, mx);
+    const float corr = __expf(m - mn);
+    m = mn;
+    float psum = 0.f, ev[2][4];
+#pragma unroll
+    for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        ev[nt][r] = __expf(sv[nt][r] - mn);
+        psum += ev[nt][r];
+      }
+    l = l * corr + rows_sum(psum);
+    const u32x4_t pf = {pack_bf16x2(ev[0][0], ev[0][1]), pack_bf16x2(ev[0][2], ev[0][3]), pack_bf16x2(ev[1][0], ev[1][1]),
+                        pack_bf16x2(ev[1][2], ev[1][3])};
+    if (__builtin_amdgcn_ballot_w64(corr != 1.f) != 0ull) {
+#pragma unroll
+      for (int t = 0; t < DT; ++t)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) oacc[t][r] *= corr;
+    }
+    const unsigned char* tr0 = vsm + (kb * 4 + (ni >> 2)) * pitchv + (ni & 3) * 8;
+#pragma unroll
+    for (int t = 0; t < DT; ++t) {
+      if (t * 16 < DV) {
+        const u32x2_t lo2 = lds_read_tr16(tr0 + t * 32);
+        const u32x2_t hi2 = lds_read_tr16(tr0 + t * 32 + 16 * pitchv);
+        const u32x4_t vf = {lo2[0], lo2[1], hi2[0], hi2[1]};
+        oacc[t] = mfma_bf16g(vf, pf, oacc[t]);
+      }
+    }
+    __syncthreads();
+  }
+  asm volatile("s_nop 15\n\ts_nop 7" ::: "memory");
+  if (!row_ok) return;
+  if (nsplit == 1) {
+    const float inv = (a.gate ? a.gate[(size_t)(row0 + tq) * a.ldg + h] : 1.f) / l;
+    float* o = a.out + (size_t)(row0 + tq) * a.ldo + (size_t)h * DV + kb * 4;
+#pragma unroll
+    for (int t = 0; t < DT; ++t)
+      if (t * 16 + kb * 4 < DV) *reinterpret_cast<f32x4_t*>(o + t * 16) = f32x4_t{oacc[t][0] * inv, oacc[t][1] * inv, oacc[t][2] * inv, oacc[t][3] * inv};
+  } else {
+    float* o = a.ws + ((size_t)split * a.rows_total + (size_t)(row0 + tq) * H + h) * (Vp + 4);
+#pragma unroll
+    for (int t = 0; t < DT; ++t)
+      if (t * 16 < Vp) *reinterpret_cast<f32x4_t*>(o + t * 16 + kb * 4) = oacc[t];
+    if (kb == 0) { o[Vp] = m; o[Vp + 1] = l; }
+  }
+}
+
+// one workgroup per (row, head): the splits' (maximum, denominator, sums) records -> the row's output
+__global__ __launch_bounds__(256) void gqa_attn_merge_kernel(float* __restrict__ out, long ldo, const float* __restrict__ ws, int nsplit,
+                                                             int rows_total, int H, int DV, int Vp, const float* __restrict__ gate, long ldg) {
+  __shared__ float wgt[1024];
+  __shared__ float red[4];
+  const int gi = blockIdx.x, t = gi / H, h = gi - t * H;
+  const size_t rec = (size_t)Vp + 4, stride = (size_t)rows_total * rec;
+  const float* base = ws + (size_t)gi * rec;
+  float mloc[4], lloc[4], mx = -INFINITY;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int s = threadIdx.x + i * 256;
+    mloc[i] = s < nsplit ? base[s * stride + Vp] : -INFINITY;
+    lloc[i] = s < nsplit ? base[s * stride + Vp + 1] : 0.f;
+    mx = fmaxf(mx, mloc[i]);
+  }
+  mx = wave_max(mx);
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = mx;
+  __syncthreads();
+  mx = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+  float den = 0.f;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int s = threadIdx.x + i * 256;
+    const float w = s < nsplit ? expf(mloc[i] - mx) : 0.f;
+    if (s < nsplit) wgt[s] = w;
+    den = __builtin_fmaf(w, lloc[i], den);
+  }
+  den = block256_sum(den, red);      // (its barriers publish wgt)
+  const float inv = (gate ? gate[(size_t)t * ldg + h] : 1.f) / den;
+  for (int r = threadIdx.x; r < DV; r += 256) {
+    float acc = 0.f;
+#pragma unroll 8
+    for (int s = 0; s < nsplit; ++s) acc = __builtin_fmaf(wgt[s], base[s * stride + r], acc);
+    out[(size_t)t * ldo + (size_t)h * DV + r] = acc * inv;
+  }
+}
+
+}  // namespace
+}  // namespace dihip
+
+using namespace dihip;
+
+extern "C" {
+
+int dihip_qkv_prep_append(void* stream, float* qkv, long ld, int q_off, int k_off, int v_off, int H, int G, int D, int DV,
+                          const void* qnorm, const void* knorm, int w_dtype, float eps, const float* freq, int rot_dims, int layout,
+                          float mag, float lam, const float* vfirst_in, float* vfirst_out, long ldvf, void* const* kspans,
+                          void* const* vspans, int span_stride, int span_len, int cache_dtype, const int32_t* tok_slot,
+                          const int32_t* tok_pos, int T) {
+  DIHIP_REQUIRE(T >= 0 && qkv && H > 0 && G > 0 && H % G == 0 && D > 0 && D <= 256 && DV > 0 && kspans && vspans && tok_slot && tok_pos &&
+                    span_stride > 0 && span_len > 0 && seq_dtype_ok(cache_dtype) && seq_dtype_ok(w_dtype), DIHIP_PARAM_ERROR,
+                "qkv_prep_append: bad argument (heads of at most 256 elements)");
+  DIHIP_REQUIRE(q_off >= 0 && k_off >= 0 && v_off >= 0 && ld >= (long)q_off + (long)H * D && ld >= (long)k_off + (long)G * D &&
+                    ld >= (long)v_off + (long)G * DV, DIHIP_PARAM_ERROR, "qkv_prep_append: columns outside the rows");
+  DIHIP_REQUIRE(rot_dims >= 0 && rot_dims <= D && rot_dims % 2 == 0 && (rot_dims == 0 || freq) && (layout == 0 || layout == 1),
+                DIHIP_PARAM_ERROR, "qkv_prep_append: bad rotation (an even number of dimensions up to the head size, layout 0 / 1)");
+  DIHIP_REQUIRE((!vfirst_in && !vfirst_out) || ldvf >= (long)G * DV, DIHIP_PARAM_ERROR, "qkv_prep_append: value rows shorter than the values");
+  if (T == 0) return DIHIP_SUCCESS;
+  PrepArgs a{qkv, ld, q_off, k_off, v_off, H, G, D, DV, qnorm, knorm, w_dtype, eps, freq, rot_dims, layout, mag, lam, vfirst_in, vfirst_out,
+             ldvf, kspans, vspans, span_stride, span_len, cache_dtype, tok_slot, tok_pos};
+  hipLaunchKernelGGL(qkv_prep_append_kernel, dim3(T), dim3(256), 0, reinterpret_cast<hipStream_t>(stream), a);
+  return launch_status();
+}
+
+static int gqa_check(const char* what, const float* out, long ldo, const float* q, long ldq, void* const* kspans, void* const* vspans,
+                     int span_stride, int span_len, const void* sink, int w_dtype, int sink_mode, const float* gate, long ldg, int H, int G,
+                     int D, int DV) {
+  DIHIP_REQUIRE(out && q && kspans && vspans && span_stride > 0 && span_len > 0 && H > 0 && G > 0 && H % G == 0 && D > 0 && DV > 0 &&
+                    ldo >= (long)H * DV && ldq >= (long)H * D && seq_dtype_ok(w_dtype), DIHIP_PARAM_ERROR, "%s: bad argument", what);
+  DIHIP_REQUIRE(sink_mode >= 0 && sink_mode <= 2 && (sink_mode != 1 || sink) && (!gate || ldg >= H), DIHIP_PARAM_ERROR,
+                "%s: bad sink mode or gate", what);
+  return DIHIP_SUCCESS;
+}
+
+int dihip_gqa_attn(void* stream, float* out, long ldo, const float* q, long ldq, void* const* kspans, void* const* vspans,
+                   int span_stride, int span_len, int cache_dtype, const void* sink, int w_dtype, int sink_mode, float softcap,
+                   const float* gate, long ldg, const int32_t* tok_slot, const int32_t* tok_pos, int T, int H, int G, int D, int DV,
+                   float scale) {
+  if (int rc = gqa_check("gqa_attn", out, ldo, q, ldq, kspans, vspans, span_stride, span_len, sink, w_dtype, sink_mode, gate, ldg, H, G, D, DV)) return rc;
+  DIHIP_REQUIRE(T >= 0 && tok_slot && tok_pos && seq_dtype_ok(cache_dtype), DIHIP_PARAM_ERROR, "gqa_attn: bad argument");
+  DIHIP_REQUIRE(D <= 256 && DV <= 512, DIHIP_EXCEED_LIMIT_ERROR, "gqa_attn: head sizes above 256 (keys) / 512 (values)");
+  if (T == 0) return DIHIP_SUCCESS;
+  GqaArgs a{out, ldo, q, ldq, kspans, vspans, span_stride, span_len, sink, w_dtype, sink_mode, softcap, gate, ldg, tok_slot, tok_pos,
+            nullptr, nullptr, nullptr, H, G, D, DV, scale, nullptr, 0};
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  auto go = [&](auto ct, auto rv) {
+    constexpr int CT = decltype(ct)::value, RV = decltype(rv)::value;
+    hipLaunchKernelGGL((gqa_attn_kernel<CT, RV>), dim3(T), dim3(256), 0, s, a);
+  };
+  auto by_v = [&](auto ct) {
+    if (DV <= 64) go(ct, std::integral_constant<int, 1>{});
+    else if (DV <= 128) go(ct, std::integral_constant<int, 2>{});
+    else if (DV <= 256) go(ct, std::integral_constant<int, 4>{});
+    else go(ct, std::integral_constant<int, 8>{});
+  };
+  if (cache_dtype == DIHIP_F32) by_v(std::integral_constant<int, DIHIP_F32>{});
+  else by_v(std::integral_constant<int, DIHIP_BF16>{});
+  return launch_status();
+}
+
+int dihip_gqa_attn_mc_supported(int D, int DV, int span_len, int cache_dtype) {
+  return cache_dtype == DIHIP_BF16 && D % 8 == 0 && DV % 8 == 0 && D >= 8 && DV >= 8 && D <= 256 && DV <= 128 && span_len % 32 == 0;
+}
+
+size_t dihip_gqa_attn_mc_workspace_bytes(int T, int H, int DV, int nsplit) {
+  return nsplit > 1 ? (size_t)nsplit * T * H * (((DV + 15) & ~15) + 4) * sizeof(float) : 0;
+}
+
+int dihip_gqa_attn_mc(void* stream, float* out, long ldo, const float* q, long ldq, void* const* kspans, void* const* vspans,
+                      int span_stride, int span_len, const void* sink, int w_dtype, int sink_mode, float softcap, const float* gate,
+                      long ldg, const int32_t* tok_pos, const int32_t* ent_slot, const int32_t* ent_row0, const int32_t* ent_count, int E,
+                      int max_count, int T, int H, int G, int D, int DV, float scale, int nsplit, void* ws, size_t ws_bytes) {
+  if (int rc = gqa_check("gqa_attn_mc", out, ldo, q, ldq, kspans, vspans, span_stride, span_len, sink, w_dtype, sink_mode, gate, ldg, H, G, D, DV)) return rc;
+  DIHIP_REQUIRE(dihip_gqa_attn_mc_supported(D, DV, span_len, DIHIP_BF16), DIHIP_PARAM_ERROR,
+                "gqa_attn_mc: head sizes %d / %d (multiples of 8 up to 256 / 128) or span_len %d (a multiple of 32) not served", D, DV, span_len);
+  DIHIP_REQUIRE(E >= 0 && T >= 0 && max_count >= 0 && tok_pos && ent_slot && ent_row0 && ent_count && ldo % 4 == 0 && ldq % 4 == 0,
+                DIHIP_PARAM_ERROR, "gqa_attn_mc: bad argument");
+  DIHIP_REQUIRE((reinterpret_cast<uintptr_t>(out) & 15u) == 0 && (reinterpret_cast<uintptr_t>(q) & 15u) == 0, DIHIP_PARAM_ERROR,
+                "gqa_attn_mc: q / out must be 16-byte aligned");
+  DIHIP_REQUIRE(nsplit >= 1 && nsplit <= 1024 && (long)E * G <= 65535, DIHIP_PARAM_ERROR, "gqa_attn_mc: bad split / portion count");
+  DIHIP_REQUIRE(ws_bytes >= dihip_gqa_attn_mc_workspace_bytes(T, H, DV, nsplit) && (nsplit == 1 || ws), DIHIP_PARAM_ERROR,
+                "gqa_attn_mc: workspace too small");
+  if (E == 0 || max_count == 0) return DIHIP_SUCCESS;
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  GqaArgs a{out, ldo, q, ldq, kspans, vspans, span_stride, span_len, sink, w_dtype, sink_mode, softcap, gate, ldg, nullptr, tok_pos,
+            ent_slot, ent_row0, ent_count, H, G, D, DV, scale, (float*)ws, T * H};
+  const int hpg = H / G, Dp = (D + 31) & ~31, Vp = (DV + 15) & ~15;
+  const dim3 grid((unsigned)(((long)max_count * hpg + 63) / 64), E * G, nsplit);
+  const size_t lds = (size_t)32 * ((Dp + 8) + (Vp + 8)) * 2;
+  auto go = [&](auto dm, auto vm) {
+    constexpr int DM = decltype(dm)::value, VM = decltype(vm)::value;
+    hipLaunchKernelGGL((gqa_attn_mc_kernel<DM, VM>), grid, dim3(256), lds, s, a);
+  };
+  auto by_v = [&](auto dm) {
+    if (DV <= 64) go(dm, std::integral_constant<int, 64>{});
+    else go(dm, std::integral_constant<int, 128>{});
+  };
+  if (D <= 64) by_v(std::integral_constant<int, 64>{});
+  else if (D <= 128) by_v(std::integral_constant<int, 128>{});
+  else by_v(std::integral_constant<int, 256>{});
+  if (nsplit > 1) hipLaunchKernelGGL(gqa_attn_merge_kernel, dim3(T * H), dim3(256), 0, s, out, ldo, (const float*)ws, nsplit, T * H, H, DV, Vp, gate, ldg);
+  return launch_status();
+}
+
+}  // extern "C"

@@ -15,7 +15,15 @@ struct LinArgs {
   void* y; long ldy, yg;
   const float* mul; long ldm;
   int T, N, K, act, act_lo, act_hi, ydt, round_ops;
+  const int32_t* seg; const int32_t* row_map;   // segmented form: group g owns the output rows seg[g] .. seg[g + 1], row r reads x row row_map[r]
 };
+
+// the rows of group g: [lo, hi)
+__device__ __forceinline__ void lin_rows(const LinArgs& a, int g, int& lo, int& hi) {
+  lo = 0; hi = a.T;
+  if (a.seg) { lo = a.seg[g]; hi = a.seg[g + 1]; }
+}
+__device__ __forceinline__ size_t lin_xrow(const LinArgs& a, int r) { return (size_t)(a.row_map ? a.row_map[r] : r); }
 
 __device__ __forceinline__ void lin_epilogue(const LinArgs& a, int g, int t, int n, float v, int wdt) {
   if (a.bias) v += ld_any(a.bias, (size_t)g * a.N + n, wdt);
@@ -32,7 +40,11 @@ __global__ __launch_bounds__(256) void linear_tile_kernel(LinArgs a) {
   __shared__ float xs[16][68];
   __shared__ float ws[16][68];
   const int tid = threadIdx.x, tx = tid & 15, ty = tid >> 4;
-  const int g = blockIdx.z, m0 = blockIdx.y * 64, n0 = blockIdx.x * 64;
+  const int g = blockIdx.z, n0 = blockIdx.x * 64;
+  int t_lo, t_hi;
+  lin_rows(a, g, t_lo, t_hi);
+  const int m0 = t_lo + blockIdx.y * 64;
+  if (m0 >= t_hi) return;
   const size_t xoff = (size_t)(g % a.xgroups) * a.xg;
   const size_t wbase = (size_t)g * a.N * a.K;
   float acc[4][4];
@@ -46,7 +58,7 @@ __global__ __launch_bounds__(256) void linear_tile_kernel(LinArgs a) {
       const int idx = tid + 256 * j, r = idx >> 4, kk = idx & 15;
       float xv = 0.f, wv = 0.f;
       if (k0 + kk < a.K) {
-        if (m0 + r < a.T) xv = load_ft<XT>(a.x, (size_t)(m0 + r) * a.ldx + xoff + k0 + kk);
+        if (m0 + r < t_hi) xv = load_ft<XT>(a.x, lin_xrow(a, m0 + r) * a.ldx + xoff + k0 + kk);
         if (n0 + r < a.N) wv = load_ft<WT>(a.w, wbase + (size_t)(n0 + r) * a.K + k0 + kk);
       }
       if (a.round_ops) { xv = ft_round<DIHIP_BF16>(xv); wv = ft_round<DIHIP_BF16>(wv); }
@@ -68,7 +80,7 @@ __global__ __launch_bounds__(256) void linear_tile_kernel(LinArgs a) {
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const int t = m0 + ty * 4 + i;
-    if (t >= a.T) continue;
+    if (t >= t_hi) continue;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int n = n0 + tx * 4 + j;
@@ -113,7 +125,11 @@ __global__ __launch_bounds__(256) void linear_mfma_kernel(LinArgs a) {
   __shared__ __attribute__((aligned(16))) uint16_t Bs[128 * LD];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1;
-  const int g = blockIdx.z, m0 = blockIdx.y * 128, n0 = blockIdx.x * 128;
+  const int g = blockIdx.z, n0 = blockIdx.x * 128;
+  int t_lo, t_hi;
+  lin_rows(a, g, t_lo, t_hi);
+  const int m0 = t_lo + blockIdx.y * 128;
+  if (m0 >= t_hi) return;
   const size_t xoff = (size_t)(g % a.xgroups) * a.xg;
   const size_t wbase = (size_t)g * a.N * a.K;
   const f32x4_t z4 = {0.f, 0.f, 0.f, 0.f};
@@ -123,11 +139,17 @@ __global__ __launch_bounds__(256) void linear_mfma_kernel(LinArgs a) {
 #pragma unroll
     for (int j = 0; j < 4; ++j) acc[i][j] = z4;
   u32x4_t ra[UN], rb[UN];
+  size_t xrow[UN];   // the x row of each of the thread's units: fixed for the whole walk
+#pragma unroll
+  for (int j = 0; j < UN; ++j) {
+    const int r = (tid + 256 * j) / UPR;
+    xrow[j] = m0 + r < t_hi ? lin_xrow(a, m0 + r) : 0;
+  }
   auto fetch = [&](int k0) {
 #pragma unroll
     for (int j = 0; j < UN; ++j) {
       const int u = tid + 256 * j, r = u / UPR, k = k0 + (u % UPR) * 8;
-      ra[j] = load8_bf16<XT, VEC>(a.x, (size_t)(m0 + r) * a.ldx + xoff + k, a.K - k, m0 + r < a.T);
+      ra[j] = load8_bf16<XT, VEC>(a.x, xrow[j] * a.ldx + xoff + k, a.K - k, m0 + r < t_hi);
       rb[j] = load8_bf16<DIHIP_BF16, VEC>(a.w, wbase + (size_t)(n0 + r) * a.K + k, a.K - k, n0 + r < a.N);
     }
   };
@@ -165,7 +187,7 @@ __global__ __launch_bounds__(256) void linear_mfma_kernel(LinArgs a) {
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         const int t = m0 + wm * 64 + i * 16 + (lane >> 4) * 4 + r;
-        if (t < a.T && n < a.N) lin_epilogue(a, g, t, n, acc[i][j][r], DIHIP_BF16);
+        if (t < t_hi && n < a.N) lin_epilogue(a, g, t, n, acc[i][j][r], DIHIP_BF16);
       }
     }
 }
@@ -185,6 +207,12 @@ __device__ __forceinline__ float dot8_bf16(const u32x4_t& w, const u32x4_t& x, f
 // K % 8 == 0 and 16-byte aligned weight rows (host-checked).
 template <int XT, bool EXACT>
 __global__ __launch_bounds__(256) void linear_skinny_kernel(LinArgs a, int t0, int tc) {
+  if (a.seg) {   // rows t0 .. of the group's own segment (block-uniform)
+    const int lo = a.seg[blockIdx.y] + t0, left = a.seg[blockIdx.y + 1] - lo;
+    if (left <= 0) return;
+    t0 = lo;
+    tc = min(tc, left);
+  }
   extern __shared__ __attribute__((aligned(16))) unsigned char xraw[];
   uint16_t* xsm = reinterpret_cast<uint16_t*>(xraw);
   float* xsf = reinterpret_cast<float*>(xraw);
@@ -211,7 +239,7 @@ __global__ __launch_bounds__(256) void linear_skinny_kernel(LinArgs a, int t0, i
 #pragma unroll 4
   for (int u = tid; u < units; u += 256) {
     const int t = u / upr, k = (u - t * upr) * 8;
-    const size_t src = (size_t)(t0 + t) * a.ldx + xoff + k;
+    const size_t src = lin_xrow(a, t0 + t) * a.ldx + xoff + k;
     float v[8];
     if constexpr (XT == DIHIP_F32) {
       const f32x4_t lo = *reinterpret_cast<const f32x4_t*>((const float*)a.x + src);
@@ -292,9 +320,10 @@ inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 
 
 using namespace dihip;
 
-extern "C" int dihip_linear(void* stream, const void* x, int x_dtype, long ldx, long x_gstride, int x_groups, const void* w,
-                            int w_dtype, const void* bias, void* y, int y_dtype, long ldy, long y_gstride, const float* mul,
-                            long ldm, int T, int N, int K, int groups, int act, int act_lo, int act_hi, int math) {
+static int linear_impl(void* stream, const void* x, int x_dtype, long ldx, long x_gstride, int x_groups, const void* w,
+                       int w_dtype, const void* bias, void* y, int y_dtype, long ldy, long y_gstride, const float* mul,
+                       long ldm, int T, int N, int K, int groups, int act, int act_lo, int act_hi, int math,
+                       const int32_t* seg, const int32_t* row_map, int seg_max_rows) {
   DIHIP_REQUIRE(T >= 0 && N > 0 && K > 0 && groups > 0 && x_groups > 0, DIHIP_PARAM_ERROR, "linear: bad shape T %d N %d K %d groups %d", T, N, K, groups);
   DIHIP_REQUIRE(seq_dtype_ok(x_dtype) && seq_dtype_ok(w_dtype) && seq_dtype_ok(y_dtype), DIHIP_PARAM_ERROR, "linear: f32 / bf16 only");
   DIHIP_REQUIRE(x && w && y, DIHIP_PARAM_ERROR, "linear: null pointer");
@@ -304,7 +333,8 @@ extern "C" int dihip_linear(void* stream, const void* x, int x_dtype, long ldx, 
   DIHIP_REQUIRE(groups <= 65535, DIHIP_PARAM_ERROR, "linear: more than 65535 groups");
   if (T == 0) return DIHIP_SUCCESS;
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
-  LinArgs a{x, ldx, x_gstride, x_groups, w, bias, y, ldy, y_gstride, mul, ldm, T, N, K, act, act_lo, act_hi, y_dtype, 0};
+  LinArgs a{x, ldx, x_gstride, x_groups, w, bias, y, ldy, y_gstride, mul, ldm, T, N, K, act, act_lo, act_hi, y_dtype, 0, seg, row_map};
+  const int Tg = seg ? (seg_max_rows < T ? seg_max_rows : T) : T;   // the most rows one group can have
   const size_t xe = x_dtype == DIHIP_F32 ? 4 : 2;
   const bool vec = w_dtype == DIHIP_BF16 && K % 8 == 0 && aligned16(w) && aligned16(x) && (ldx * xe) % 16 == 0 &&
                    (x_gstride * xe) % 16 == 0;
@@ -312,9 +342,9 @@ extern "C" int dihip_linear(void* stream, const void* x, int x_dtype, long ldx, 
   if (math == DIHIP_MATH_F32_STREAM) {
     // f32 products of unrounded rows; few rows stream the weight once (a row's sum then runs in the lanes' order, not k ascending)
     const int tmax = K <= 4096 ? 4 : (K <= 8192 ? 2 : 1);
-    if (T <= 4 * tmax && vec && !no_skinny && K <= 16384) {
-      for (int t0 = 0; t0 < T; t0 += tmax) {
-        const int tc = T - t0 < tmax ? T - t0 : tmax;
+    if (Tg <= 4 * tmax && vec && !no_skinny && K <= 16384) {
+      for (int t0 = 0; t0 < Tg; t0 += tmax) {
+        const int tc = Tg - t0 < tmax ? Tg - t0 : tmax;
         const dim3 grid((N + 7) / 8, groups);
         if (x_dtype == DIHIP_F32) hipLaunchKernelGGL((linear_skinny_kernel<DIHIP_F32, true>), grid, dim3(256), (size_t)tc * K * 4, s, a, t0, tc);
         else hipLaunchKernelGGL((linear_skinny_kernel<DIHIP_BF16, true>), grid, dim3(256), (size_t)tc * K * 4, s, a, t0, tc);
@@ -325,16 +355,16 @@ extern "C" int dihip_linear(void* stream, const void* x, int x_dtype, long ldx, 
   }
   if (math == DIHIP_MATH_BF16 && w_dtype == DIHIP_BF16) {
     const int tmax = K <= 8192 ? 4 : (K <= 16384 ? 2 : 1);  // rows whose bf16 copy fits 64 KB of LDS
-    if (T <= 4 * tmax && vec && !no_skinny && K <= 32768) {
-      for (int t0 = 0; t0 < T; t0 += tmax) {
-        const int tc = T - t0 < tmax ? T - t0 : tmax;
+    if (Tg <= 4 * tmax && vec && !no_skinny && K <= 32768) {
+      for (int t0 = 0; t0 < Tg; t0 += tmax) {
+        const int tc = Tg - t0 < tmax ? Tg - t0 : tmax;
         const dim3 grid((N + 7) / 8, groups);
         if (x_dtype == DIHIP_F32) hipLaunchKernelGGL((linear_skinny_kernel<DIHIP_F32, false>), grid, dim3(256), (size_t)tc * K * 2, s, a, t0, tc);
         else hipLaunchKernelGGL((linear_skinny_kernel<DIHIP_BF16, false>), grid, dim3(256), (size_t)tc * K * 2, s, a, t0, tc);
       }
       return launch_status();
     }
-    const dim3 grid((N + 127) / 128, (T + 127) / 128, groups);
+    const dim3 grid((N + 127) / 128, (Tg + 127) / 128, groups);
     DIHIP_REQUIRE(grid.y <= 65535, DIHIP_PARAM_ERROR, "linear: too many rows for one launch");
     if (x_dtype == DIHIP_F32) {
       if (vec) hipLaunchKernelGGL((linear_mfma_kernel<DIHIP_F32, true>), grid, dim3(256), 0, s, a);
@@ -346,11 +376,27 @@ extern "C" int dihip_linear(void* stream, const void* x, int x_dtype, long ldx, 
     return launch_status();
   }
   a.round_ops = math == DIHIP_MATH_BF16;
-  const dim3 grid((N + 63) / 64, (T + 63) / 64, groups);
+  const dim3 grid((N + 63) / 64, (Tg + 63) / 64, groups);
   DIHIP_REQUIRE(grid.y <= 65535, DIHIP_PARAM_ERROR, "linear: too many rows for one launch");
   if (x_dtype == DIHIP_F32 && w_dtype == DIHIP_F32) hipLaunchKernelGGL((linear_tile_kernel<DIHIP_F32, DIHIP_F32>), grid, dim3(256), 0, s, a);
   else if (x_dtype == DIHIP_F32) hipLaunchKernelGGL((linear_tile_kernel<DIHIP_F32, DIHIP_BF16>), grid, dim3(256), 0, s, a);
   else if (w_dtype == DIHIP_F32) hipLaunchKernelGGL((linear_tile_kernel<DIHIP_BF16, DIHIP_F32>), grid, dim3(256), 0, s, a);
   else hipLaunchKernelGGL((linear_tile_kernel<DIHIP_BF16, DIHIP_BF16>), grid, dim3(256), 0, s, a);
   return launch_status();
+}
+
+extern "C" int dihip_linear(void* stream, const void* x, int x_dtype, long ldx, long x_gstride, int x_groups, const void* w,
+                            int w_dtype, const void* bias, void* y, int y_dtype, long ldy, long y_gstride, const float* mul,
+                            long ldm, int T, int N, int K, int groups, int act, int act_lo, int act_hi, int math) {
+  return linear_impl(stream, x, x_dtype, ldx, x_gstride, x_groups, w, w_dtype, bias, y, y_dtype, ldy, y_gstride, mul, ldm, T, N, K, groups,
+                     act, act_lo, act_hi, math, nullptr, nullptr, 0);
+}
+
+extern "C" int dihip_linear_segmented(void* stream, const void* x, int x_dtype, long ldx, const void* w, int w_dtype, const void* bias,
+                                      void* y, int y_dtype, long ldy, int R, int N, int K, int groups, const int32_t* seg,
+                                      const int32_t* row_map, int seg_max_rows, int act, int math) {
+  DIHIP_REQUIRE(seg && seg_max_rows >= 0, DIHIP_PARAM_ERROR, "linear_segmented: no segment table");
+  if (seg_max_rows == 0) return DIHIP_SUCCESS;
+  return linear_impl(stream, x, x_dtype, ldx, 0, 1, w, w_dtype, bias, y, y_dtype, ldy, 0, nullptr, 0, R, N, K, groups, act, 0,
+                     act ? groups * N : 0, math, seg, row_map, seg_max_rows);
 }

@@ -120,6 +120,32 @@ __global__ __launch_bounds__(256) void norm_residual_mix_kernel(float* x_out, co
   }
 }
 
+// The norm without statistics and the parallel residual step: x_out = x_in + (a + b), h = tanh(alpha * x_out) * w + bias.
+// row_idx: h[i] is the norm of row row_idx[i] (x_out is then not written).
+template <int WT>
+__global__ __launch_bounds__(256) void add_dyt_kernel(float* x_out, const float* x_in, const float* __restrict__ a, long lda,
+                                                      const float* __restrict__ b, long ldb, const int32_t* __restrict__ row_idx, float alpha,
+                                                      const void* __restrict__ w, const void* __restrict__ bias, float* __restrict__ h,
+                                                      uint16_t* __restrict__ h16, int K) {
+  const int i = blockIdx.x;
+  const size_t r = row_idx ? (size_t)row_idx[i] : (size_t)i;
+#pragma unroll 4
+  for (int k = threadIdx.x; k < K; k += 256) {
+    float v = x_in[r * K + k];
+    if (a) {
+      float s = a[r * lda + k];
+      if (b) s += b[r * ldb + k];
+      v += s;
+    }
+    if (x_out) x_out[r * K + k] = v;
+    if (w) {
+      const float y = tanhf(alpha * v) * load_ft<WT>(w, k) + load_ft<WT>(bias, k);
+      if (h) h[(size_t)i * K + k] = y;
+      if (h16) h16[(size_t)i * K + k] = (uint16_t)f32_to_bf16_bits(y);
+    }
+  }
+}
+
 // ------------------------------------------------------------------------------------------------ latent attention
 // One workgroup per row, its 4 waves take the heads in turn.  A wave walks the row's window in chunks of 64 keys: lane j
 // scores key j (f32 dot over the R latent elements, r ascending), the chunk joins the running softmax (which starts at
@@ -404,6 +430,17 @@ int dihip_norm_residual_mix(void* stream, float* x_out, const float* x_in, const
   float* top = n_mix > 0 ? stack + (size_t)(n_mix - 1) * stack_stride : nullptr;
   if (w_dtype == DIHIP_F32) hipLaunchKernelGGL(norm_residual_mix_kernel<DIHIP_F32>, dim3(T), dim3(256), 0, reinterpret_cast<hipStream_t>(stream), x_out, x_in, m, ldm, gamma, eps, top, stack, stack_stride, mix_w, n_mix, x_mix, (uint16_t*)next16, K);
   else hipLaunchKernelGGL(norm_residual_mix_kernel<DIHIP_BF16>, dim3(T), dim3(256), 0, reinterpret_cast<hipStream_t>(stream), x_out, x_in, m, ldm, gamma, eps, top, stack, stack_stride, mix_w, n_mix, x_mix, (uint16_t*)next16, K);
+  return launch_status();
+}
+
+int dihip_add_dyt(void* stream, float* x_out, const float* x_in, const float* a, long lda, const float* b, long ldb, const int32_t* row_idx,
+                  float alpha, const void* w, const void* bias, int w_dtype, float* h, void* h16, int M, int K) {
+  DIHIP_REQUIRE(M >= 0 && K > 0 && x_in && (!a || lda >= K) && (!b || (a && ldb >= K)) && (!w || bias) && (!row_idx || !x_out) &&
+                    seq_dtype_ok(w_dtype), DIHIP_PARAM_ERROR, "add_dyt: bad argument");
+  if (M == 0) return DIHIP_SUCCESS;
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  if (w_dtype == DIHIP_F32) hipLaunchKernelGGL(add_dyt_kernel<DIHIP_F32>, dim3(M), dim3(256), 0, s, x_out, x_in, a, lda, b, ldb, row_idx, alpha, w, bias, h, (uint16_t*)h16, K);
+  else hipLaunchKernelGGL(add_dyt_kernel<DIHIP_BF16>, dim3(M), dim3(256), 0, s, x_out, x_in, a, lda, b, ldb, row_idx, alpha, w, bias, h, (uint16_t*)h16, K);
   return launch_status();
 }
 

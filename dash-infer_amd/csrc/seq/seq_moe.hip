@@ -1,0 +1,133 @@
+// seq_moe.hip -- routing and glue of the mixture-of-experts feed-forward (the expert products are dihip_linear_segmented):
+//   moe_route      per token: the `top` experts of largest router logit (ties: the lower index), weights = softmax over the
+//                  chosen logits alone, f32
+//   moe_sort       the (token, choice) pairs grouped by expert in a fixed order: segment bounds per expert, the token each
+//                  sorted row reads, and where each pair went
+//   moe_glu        the experts' activation on [gate | up] rows
+//   moe_combine    out[t] = sum over the token's choices, in order, of weight * the expert's output row
+#include "seq_common.h"
+
+namespace dihip {
+namespace {
+
+__global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict__ logits, long ldl, int32_t* __restrict__ ids,
+                                                        float* __restrict__ wts, int T, int E, int top) {
+  const int t = blockIdx.x * 256 + threadIdx.x;
+  if (t >= T) return;
+  const float* z = logits + (size_t)t * ldl;
+  float best[16];
+  int bi[16];
+  for (int k = 0; k < top; ++k) {
+    float bv = -INFINITY;
+    int bx = -1;
+    for (int e = 0; e < E; ++e) {
+      bool used = false;
+      for (int j = 0; j < k; ++j) used |= bi[j] == e;
+      const float v = z[e];
+      if (!used && (bx < 0 || v > bv)) { bv = v; bx = e; }
+    }
+    best[k] = bv; bi[k] = bx;
+  }
+  float den = 0.f;
+  const float zmax = best[0];
+  for (int k = 0; k < top; ++k) { best[k] = expf(best[k] - zmax); den += best[k]; }
+  for (int k = 0; k < top; ++k) {
+    ids[(size_t)t * top + k] = bi[k];
+    wts[(size_t)t * top + k] = best[k] / den;
+  }
+}
+
+// block e: how many pairs chose expert e
+__global__ __launch_bounds__(256) void moe_count_kernel(const int32_t* __restrict__ ids, int R, int32_t* __restrict__ counts) {
+  __shared__ int red[4];
+  const int e = blockIdx.x;
+  int c = 0;
+  for (int r = threadIdx.x; r < R; r += 256) c += ids[r] == e;
+  for (int o = 32; o > 0; o >>= 1) c += __shfl_xor(c, o);
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = c;
+  __syncthreads();
+  if (threadIdx.x == 0) counts[e] = red[0] + red[1] + red[2] + red[3];
+}
+
+// block e: its pairs in ascending pair order -> sorted rows seg[e] ..; thread i scans the pairs [i * per, (i + 1) * per)
+__global__ __launch_bounds__(256) void moe_place_kernel(const int32_t* __restrict__ ids, int R, int top, int E, const int32_t* __restrict__ counts,
+                                                        int32_t* __restrict__ seg, int32_t* __restrict__ src_row, int32_t* __restrict__ dst) {
+  __shared__ int scan[256];
+  const int e = blockIdx.x, tid = threadIdx.x;
+  const int per = (R + 255) / 256, lo = min(R, tid * per), hi = min(R, lo + per);
+  int c = 0;
+  for (int r = lo; r < hi; ++r) c += ids[r] == e;
+  scan[tid] = c;
+  __syncthreads();
+  int base = 0;
+  for (int x = 0; x < e; ++x) base += counts[x];
+  if (tid == 0) {
+    seg[e] = base;
+    if (e == E - 1) seg[E] = base + counts[e];
+  }
+  int before = 0;
+  for (int x = 0; x < tid; ++x) before += scan[x];
+  int pos = base + before;
+  for (int r = lo; r < hi; ++r)
+    if (ids[r] == e) {
+      src_row[pos] = r / top;
+      dst[r] = pos;
+      ++pos;
+    }
+}
+
+__global__ __launch_bounds__(256) void moe_glu_kernel(void* __restrict__ y, int ydt, long ldy, const float* __restrict__ gu, long ldgu, int F,
+                                                      float limit, float slope) {
+  const int r = blockIdx.x;
+  for (int c = threadIdx.x; c < F; c += 256) {
+    const float g = fminf(gu[(size_t)r * ldgu + c], limit);
+    const float u = fminf(fmaxf(gu[(size_t)r * ldgu + F + c], -limit), limit);
+    st_any(y, (size_t)r * ldy + c, ydt, g * (1.f / (1.f + expf(-slope * g))) * (u + 1.f));
+  }
+}
+
+__global__ __launch_bounds__(256) void moe_combine_kernel(float* __restrict__ out, long ldo, const float* __restrict__ rows, long ldr,
+                                                          const int32_t* __restrict__ dst, const float* __restrict__ wts, int top, int K) {
+  const int t = blockIdx.x;
+  for (int c = threadIdx.x; c < K; c += 256) {
+    float acc = 0.f;
+    for (int k = 0; k < top; ++k) acc = __builtin_fmaf(wts[(size_t)t * top + k], rows[(size_t)dst[(size_t)t * top + k] * ldr + c], acc);
+    out[(size_t)t * ldo + c] = acc;
+  }
+}
+
+}  // namespace
+}  // namespace dihip
+
+using namespace dihip;
+
+extern "C" {
+
+int dihip_seq_moe_route(void* stream, const float* logits, long ldl, int32_t* ids, float* wts, int32_t* counts, int32_t* seg, int32_t* src_row,
+                    int32_t* dst, int T, int E, int top) {
+  DIHIP_REQUIRE(T >= 0 && E > 0 && top > 0 && top <= E && top <= 16 && E <= 65535 && logits && ids && wts && counts && seg && src_row && dst &&
+                    ldl >= E, DIHIP_PARAM_ERROR, "moe_route: bad argument (at most 16 choices per token)");
+  if (T == 0) return DIHIP_SUCCESS;
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  hipLaunchKernelGGL(moe_route_kernel, dim3((T + 255) / 256), dim3(256), 0, s, logits, ldl, ids, wts, T, E, top);
+  hipLaunchKernelGGL(moe_count_kernel, dim3(E), dim3(256), 0, s, ids, T * top, counts);
+  hipLaunchKernelGGL(moe_place_kernel, dim3(E), dim3(256), 0, s, ids, T * top, top, E, counts, seg, src_row, dst);
+  return launch_status();
+}
+
+int dihip_seq_moe_glu(void* stream, void* y, int y_dtype, long ldy, const float* gu, long ldgu, int R, int F, float limit, float slope) {
+  DIHIP_REQUIRE(R >= 0 && F > 0 && y && gu && ldy >= F && ldgu >= 2 * (long)F && seq_dtype_ok(y_dtype), DIHIP_PARAM_ERROR, "moe_glu: bad argument");
+  if (R == 0) return DIHIP_SUCCESS;
+  hipLaunchKernelGGL(moe_glu_kernel, dim3(R), dim3(256), 0, reinterpret_cast<hipStream_t>(stream), y, y_dtype, ldy, gu, ldgu, F, limit, slope);
+  return launch_status();
+}
+
+int dihip_seq_moe_combine(void* stream, float* out, long ldo, const float* rows, long ldr, const int32_t* dst, const float* wts, int T, int top,
+                      int K) {
+  DIHIP_REQUIRE(T >= 0 && top > 0 && K > 0 && out && rows && dst && wts && ldo >= K && ldr >= K, DIHIP_PARAM_ERROR, "moe_combine: bad argument");
+  if (T == 0) return DIHIP_SUCCESS;
+  hipLaunchKernelGGL(moe_combine_kernel, dim3(T), dim3(256), 0, reinterpret_cast<hipStream_t>(stream), out, ldo, rows, ldr, dst, wts, top, K);
+  return launch_status();
+}
+
+}  // extern "C"

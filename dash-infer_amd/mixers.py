@@ -7,6 +7,14 @@ to rows of the same shape, reading and updating what its sequences left in the s
   GatedLinearRecurrence  two-branch recurrent block: gelu branch x (short causal convolution -> block-diagonal gates ->
                          real-gated diagonal recurrence), f32 state and convolution tail per slot
   DenseMlp               down(act(up(h)))
+  GroupedQueryAttention  causal attention over paged key and value caches with fewer key/value heads than query heads; options:
+                         unit-RMS norm of queries and keys, rotary positions (paired or half-split layout, part of the head,
+                         frequencies rescaled for longer contexts), biases, a sink logit (per head or the constant 0), a tanh cap
+                         on the scores, a sigmoid gate per head, values mixed with those of an earlier layer of the same step
+  GatedLinearAttention   linear attention with a decay per key channel and a matrix state per head (f32, per slot), unit-RMS
+                         norm per head, silu output gate
+  GatedMlp               down(act(gate(h)) * up(h))
+  ExpertMlp              top-k routed experts with clamped gated units, weights = softmax over the chosen logits
 Matrix products run in ctx.math (seq_ops.MATH_F32 / MATH_BF16); norms, scores, gates of the recurrence, decays and
 state are f32 in both.
 """
@@ -25,6 +33,7 @@ class StepContext:
         self.math, self.eps = math, eps
         self.max_count, self.max_pos = T, 0     # host numbers: the largest portion and the last position of the step
         self.taps = None    # layer index -> [T, .] intermediate (diagnostics; None: off)
+        self.shared = {}    # what a layer leaves for later layers of the SAME step (values to be mixed in)
 
     def act_buffer(self, n, dtype=None):
         """[T, n] for an activation that only a product reads: bf16 under bf16 products (the product would round it anyway), else f32"""
@@ -110,3 +119,158 @@ class DenseMlp:
     def __call__(self, ctx, h, h16=None):
         act = so.linear(h16 if h16 is not None else h, self.up, act=self.act, math=ctx.math, out=ctx.act_buffer(self.up.shape[0]))
         return so.linear(act, self.down, math=ctx.math)
+
+
+def rotary_frequencies(dims, base, scaling=None):
+    """frequency per rotated pair (f32 tensor [dims / 2], computed in f64) and the magnitude of cos and sin.  scaling: None or
+    {factor, original, fast, slow}: pairs that turn fewer than `slow` times over `original` positions are slowed down by
+    `factor`, pairs that turn more than `fast` times are kept, a linear ramp over the pair index between; the magnitude grows
+    with 0.1 ln(factor) + 1."""
+    import math
+    f = [float(base) ** (-2.0 * i / dims) for i in range(dims // 2)]
+    mag = 1.0
+    if scaling:
+        factor, orig = float(scaling["factor"]), float(scaling["original"])
+        where = lambda turns: dims * math.log(orig / (2.0 * math.pi * turns)) / (2.0 * math.log(float(base)))
+        lo = max(math.floor(where(float(scaling["fast"]))), 0)
+        hi = min(math.ceil(where(float(scaling["slow"]))), dims - 1)
+        for i in range(dims // 2):
+            ramp = min(max((i - lo) / max(hi - lo, 0.001), 0.0), 1.0)
+            f[i] = f[i] / factor * ramp + f[i] * (1.0 - ramp)
+        mag = 0.1 * math.log(factor) + 1.0
+    return torch.tensor(f, dtype=torch.float64).to(torch.float32), mag
+
+
+class GroupedQueryAttention:
+    LAYOUTS = {"pairs": 0, "halves": 1}
+
+    def __init__(self, key, heads, kv_heads, dim, vdim, scale, w, state, cache_dtype, rot_dims=0, rot_base=10000.0, rot_layout="pairs",
+                 rot_scaling=None, qk_norm=False, sink=None, softcap=None, head_gate=False, value_mix=None):
+        """w: q [heads*dim, width], k [kv_heads*dim, width], v [kv_heads*vdim, width] (+ q.b / k.b / v.b where present), q.norm /
+        k.norm [dim] (qk_norm), g [heads, width] (head_gate), o [width, heads*vdim].  sink: None, "zero" or a tensor [heads].
+        value_mix: None, ("source", name): this layer's values are kept under `name` for the step, or ("mix", name, lam):
+        v <- (1 - lam) v + lam * the values kept under `name`."""
+        assert heads % kv_heads == 0
+        self.H, self.G, self.D, self.V, self.scale = heads, kv_heads, dim, vdim, float(scale)
+        dev = w["q"].device
+        parts = [w["q"], w["k"], w["v"]] + ([w["g"]] if head_gate else [])
+        n = sum(p.shape[0] for p in parts)
+        if n % 4:    # rows of the product's output stay 16-byte aligned for the attention kernels: zero weight rows at the end
+            parts.append(torch.zeros(4 - n % 4, w["q"].shape[1], dtype=w["q"].dtype, device=dev))
+        self.w_in = torch.cat(parts, 0).contiguous()
+        self.k_lo, self.v_lo = heads * dim, (heads + kv_heads) * dim
+        self.g_lo = self.v_lo + kv_heads * vdim
+        self.n_in = self.w_in.shape[0]
+        self.head_gate = head_gate
+        self.b_in = None
+        if "q.b" in w or "k.b" in w or "v.b" in w:
+            zero = lambda n: torch.zeros(n, dtype=self.w_in.dtype, device=dev)
+            b = [w.get("q.b", zero(heads * dim)), w.get("k.b", zero(kv_heads * dim)), w.get("v.b", zero(kv_heads * vdim))]
+            b = torch.cat(b + ([zero(heads)] if head_gate else []), 0)
+            self.b_in = torch.cat([b, zero(self.n_in - b.shape[0])], 0).contiguous()
+        self.q_norm, self.k_norm = (w["q.norm"].contiguous(), w["k.norm"].contiguous()) if qk_norm else (None, None)
+        self.rot_dims, self.layout = int(rot_dims), self.LAYOUTS[rot_layout]
+        assert self.rot_dims % 2 == 0 and self.rot_dims <= dim
+        self.freq, self.mag = None, 1.0
+        if self.rot_dims:
+            f, self.mag = rotary_frequencies(self.rot_dims, rot_base, rot_scaling)
+            self.freq = f.to(dev)
+        self.sink_mode, self.sink = so.SINK_NONE, None
+        if isinstance(sink, str):
+            assert sink == "zero"
+            self.sink_mode = so.SINK_ZERO
+        elif sink is not None:
+            self.sink_mode, self.sink = so.SINK_PER_HEAD, sink.contiguous()
+        self.softcap = float(softcap or 0.0)
+        self.value_mix = value_mix
+        self.o = w["o"].contiguous()
+        assert self.o.shape[1] == heads * vdim and w["q"].shape[0] == heads * dim and w["k"].shape[0] == kv_heads * dim
+        self.ktable = state.add_span_cache(key + ".k", kv_heads * dim, cache_dtype)
+        self.vtable = state.add_span_cache(key + ".v", kv_heads * vdim, cache_dtype)
+        self.mc = so.gqa_attn_mc_supported(self.ktable, self.vtable, kv_heads) and self.n_in % 4 == 0 and (heads * dim) % 4 == 0
+
+    def __call__(self, ctx, h, h16=None):
+        H, G, D, V = self.H, self.G, self.D, self.V
+        a = so.linear(h16 if h16 is not None else h, self.w_in, self.b_in, act="sigmoid" if self.head_gate else None,
+                      act_cols=(self.g_lo, self.n_in), math=ctx.math)                                        # [q | k | v | gate]
+        vin = vout = None
+        lam = 0.0
+        if self.value_mix is not None:
+            if self.value_mix[0] == "source":
+                vout = ctx.shared[self.value_mix[1]] = torch.empty(ctx.T, G * V, dtype=torch.float32, device=a.device)
+            else:
+                vin, lam = ctx.shared[self.value_mix[1]], self.value_mix[2]
+                assert vin.shape[1] == G * V, "mixed values must have this layer's shape"
+        so.qkv_prep_append(a, 0, self.k_lo, self.v_lo, H, G, D, V, self.q_norm, self.k_norm, ctx.eps, self.freq, self.rot_dims, self.layout,
+                           self.mag, lam, vin, vout, self.ktable, self.vtable, ctx.tok_slot, ctx.tok_pos)
+        gate = a[:, self.g_lo:] if self.head_gate else None
+        if ctx.math == so.MATH_BF16 and self.mc:
+            o = so.gqa_attn_mc(a, self.ktable, self.vtable, ctx.tok_pos, ctx.ent_slot, ctx.ent_row0, ctx.ent_count, ctx.max_count, ctx.max_pos,
+                               H, G, D, V, self.scale, self.sink, self.sink_mode, self.softcap, gate)
+        else:
+            o = so.gqa_attn(a, self.ktable, self.vtable, ctx.tok_slot, ctx.tok_pos, H, G, D, V, self.scale, self.sink, self.sink_mode,
+                            self.softcap, gate)
+        return so.linear(o, self.o, math=ctx.math)
+
+
+class GatedLinearAttention:
+    def __init__(self, key, heads, dim, vdim, tau, w, state, q_scale=None):
+        """w: q / k [heads*dim, width], v / g [heads*vdim, width], a1 [rank, width], a2 [heads*dim, rank], a2.b, norm [vdim],
+        o [width, heads*vdim].  Decay per key channel: sigmoid(a2 (a1 h) + a2.b)^(1 / tau)."""
+        self.H, self.D, self.V, self.tau = heads, dim, vdim, float(tau)
+        self.q_scale = float(q_scale) if q_scale is not None else dim ** -0.5
+        self.w_in = torch.cat([w["q"], w["k"], w["v"], w["g"], w["a1"]], 0).contiguous()
+        hd, hv = heads * dim, heads * vdim
+        self.k_lo, self.v_lo, self.g_lo, self.a_lo = hd, 2 * hd, 2 * hd + hv, 2 * hd + 2 * hv
+        self.a2, self.a2_b = w["a2"].contiguous(), w["a2.b"].contiguous()
+        self.norm, self.o = w["norm"].contiguous(), w["o"].contiguous()
+        assert w["q"].shape[0] == hd and w["v"].shape[0] == hv and self.a2.shape == (hd, w["a1"].shape[0]) and self.o.shape[1] == hv
+        self.S = state.add_state(key + ".S", (heads, dim, vdim))
+
+    def __call__(self, ctx, h, h16=None):
+        H, D, V = self.H, self.D, self.V
+        a = so.linear(h16 if h16 is not None else h, self.w_in, act="silu", act_cols=(self.g_lo, self.a_lo), math=ctx.math)   # [q | k | v | silu g | a1 h]
+        z = so.linear(a[:, self.a_lo:], self.a2, self.a2_b, math=ctx.math)
+        o = so.gla(a, a[:, self.k_lo:], a[:, self.v_lo:], z, self.q_scale, self.tau, self.S, ctx.ent_slot, ctx.ent_row0, ctx.ent_count,
+                   ctx.max_count, H, D, V)
+        on = so.head_rmsnorm_mul(o, self.norm, ctx.eps, H, V, mul=a[:, self.g_lo: self.a_lo], out=ctx.act_buffer(H * V))
+        return so.linear(on, self.o, math=ctx.math)
+
+
+class GatedMlp:
+    def __init__(self, gate, up, down, act):
+        self.gate, self.up, self.down, self.act = gate.contiguous(), up.contiguous(), down.contiguous(), act
+
+    def __call__(self, ctx, h, h16=None):
+        x = h16 if h16 is not None else h
+        u = so.linear(x, self.up, math=ctx.math)
+        g = so.linear(x, self.gate, act=self.act, mul=u, math=ctx.math, out=ctx.act_buffer(self.gate.shape[0]))   # act(gate h) * (up h)
+        return so.linear(g, self.down, math=ctx.math)
+
+
+class ExpertMlp:
+    GLU_SLOPE = 1.702    # g * sigmoid(1.702 g): the sigmoid form of gelu
+
+    def __init__(self, router, router_b, gates, ups, downs, top, limit):
+        """gates / ups [ff, width] and downs [width, ff] per expert; an expert is down(glu(min(gate h, limit), clamp(up h, +-limit)))"""
+        self.E, self.top, self.limit = len(gates), int(top), float(limit)
+        self.router, self.router_b = router.contiguous(), router_b.contiguous()
+        self.F = gates[0].shape[0]
+        self.w_gu = torch.stack([torch.cat([g, u], 0) for g, u in zip(gates, ups)]).contiguous()    # [E, 2 ff, width]
+        self.w_down = torch.stack(list(downs)).contiguous()                                          # [E, width, ff]
+        assert self.router.shape[0] == self.E and 0 < self.top <= self.E
+
+    def __call__(self, ctx, h, h16=None):
+        x = h16 if h16 is not None else h
+        T, R = ctx.T, ctx.T * self.top
+        logits = so.linear(x, self.router, self.router_b, math=so.MATH_F32 if ctx.math == so.MATH_F32 else so.MATH_F32_STREAM)
+        _, wts, seg, src_row, dst = so.moe_route(logits, self.top)
+        gu = so.linear_segmented(x, self.w_gu, seg, src_row, T, R, math=ctx.math)
+        y = so.moe_glu(gu, self.F, self.limit, self.GLU_SLOPE, ctx_rows(ctx, R, self.F))
+        d = so.linear_segmented(y, self.w_down, seg, None, T, R, math=ctx.math)
+        return so.moe_combine(d, dst, wts, T, self.top)
+
+
+def ctx_rows(ctx, rows, n):
+    """[rows, n] for an activation that only a product reads (see StepContext.act_buffer)"""
+    return torch.empty(rows, n, dtype=torch.bfloat16 if ctx.math == so.MATH_BF16 else torch.float32, device=ctx.ids.device)

@@ -12,6 +12,7 @@ from . import seq_capi
 from .seq_capi import ACT, MATH_BF16, MATH_F32, MATH_F32_STREAM, check, lib
 
 _DT = {torch.float32: seq_capi.F32, torch.bfloat16: seq_capi.BF16}
+F32_CODE = seq_capi.F32
 
 
 def dt(t):
@@ -158,4 +159,141 @@ def gated_recurrence(r, i, u, y, lam, decay, state, ent_slot, ent_row0, ent_coun
     check(lib().dihip_gated_recurrence(stream(), ptr(o), _rows(o), ptr(r), ptr(i), _rows(r), ptr(u), _rows(u), ptr(y), _rows(y), ptr(lam),
                                        dt(lam), float(decay), ptr(state), ptr(ent_slot), ptr(ent_row0), ptr(ent_count),
                                        ent_slot.shape[0], Cn), "dihip_gated_recurrence")
+    return o
+
+
+def linear_segmented(x, w, seg, row_map, seg_max_rows, R, bias=None, out=None, act=None, math=MATH_F32):
+    """rows grouped by owner: w [groups, N, K]; output row r (seg[g] <= r < seg[g + 1]) = x[row_map[r]] . w[g]^T (+ bias[g]);
+    seg_max_rows: a host-known bound on one group's rows -> [R, N] f32"""
+    groups, N, K = w.shape
+    assert x.shape[1] == K and w.is_contiguous() and seg.dtype == torch.int32 and seg.shape[0] == groups + 1
+    y = out if out is not None else torch.empty(R, N, dtype=torch.float32, device=x.device)
+    assert y.shape == (R, N)
+    check(lib().dihip_linear_segmented(stream(), ptr(x), dt(x), _rows(x), ptr(w), dt(w), ptr(bias), ptr(y), dt(y), _rows(y), R, N, K, groups,
+                                       ptr(seg), ptr(row_map), int(seg_max_rows), ACT[act], math), "dihip_linear_segmented")
+    return y
+
+
+def add_dyt(x_in, a=None, b=None, norm=None, x_out=None, row_idx=None, want16=False):
+    """x_out = x_in + (a + b);  h = tanh(alpha * x_out) * w + bias for norm = (alpha, w, bias) -> (h f32, h16 bf16 or None)"""
+    K = x_in.shape[1]
+    M = x_in.shape[0] if row_idx is None else row_idx.shape[0]
+    assert x_in.is_contiguous() and x_in.dtype == torch.float32 and (x_out is None or x_out.is_contiguous())
+    h = h16 = None
+    alpha, w, bias = 0.0, None, None
+    if norm is not None:
+        alpha, w, bias = norm
+        if want16:
+            h16 = torch.empty(M, K, dtype=torch.bfloat16, device=x_in.device)
+        else:
+            h = torch.empty(M, K, dtype=torch.float32, device=x_in.device)
+    check(lib().dihip_add_dyt(stream(), ptr(x_out), ptr(x_in), ptr(a), _rows(a) if a is not None else 0, ptr(b), _rows(b) if b is not None else 0,
+                              ptr(row_idx), float(alpha), ptr(w), ptr(bias), dt(w) if w is not None else F32_CODE, ptr(h), ptr(h16), M, K),
+          "dihip_add_dyt")
+    return h, h16
+
+
+def qkv_prep_append(a, q_off, k_off, v_off, H, G, D, DV, qnorm, knorm, eps, freq, rot_dims, layout, mag, lam, vfirst_in, vfirst_out,
+                    ktable, vtable, tok_slot, tok_pos):
+    """norm + rotation of the q / k columns of the rows a (q in place), value mixing, append of k and v to their pages"""
+    T = a.shape[0]
+    assert a.dtype == torch.float32 and ktable.row_elems == G * D and vtable.row_elems == G * DV and ktable.dtype == vtable.dtype
+    vf = vfirst_in if vfirst_in is not None else vfirst_out
+    wn = qnorm if qnorm is not None else knorm
+    check(lib().dihip_qkv_prep_append(stream(), ptr(a), _rows(a), q_off, k_off, v_off, H, G, D, DV, ptr(qnorm), ptr(knorm),
+                                      dt(wn) if wn is not None else F32_CODE, float(eps), ptr(freq), int(rot_dims), int(layout), float(mag),
+                                      float(lam), ptr(vfirst_in), ptr(vfirst_out), _rows(vf) if vf is not None else 0, ptr(ktable.ptrs),
+                                      ptr(vtable.ptrs), ktable.max_spans, ktable.span_len, _DT[ktable.dtype], ptr(tok_slot), ptr(tok_pos), T),
+          "dihip_qkv_prep_append")
+
+
+SINK_NONE, SINK_PER_HEAD, SINK_ZERO = 0, 1, 2
+
+
+def gqa_attn(q, ktable, vtable, tok_slot, tok_pos, H, G, D, DV, scale, sink=None, sink_mode=SINK_NONE, softcap=0.0, gate=None, out=None):
+    """q: f32 [T, >= H * D] rows (a column slice is fine); gate: f32 [T, >= H] or None -> f32 [T, H * DV]"""
+    T = q.shape[0]
+    o = out if out is not None else torch.empty(T, H * DV, dtype=torch.float32, device=q.device)
+    check(lib().dihip_gqa_attn(stream(), ptr(o), _rows(o), ptr(q), _rows(q), ptr(ktable.ptrs), ptr(vtable.ptrs), ktable.max_spans, ktable.span_len,
+                               _DT[ktable.dtype], ptr(sink), dt(sink) if sink is not None else F32_CODE, int(sink_mode), float(softcap or 0.0),
+                               ptr(gate), _rows(gate) if gate is not None else 0, ptr(tok_slot), ptr(tok_pos), T, H, G, D, DV, float(scale)),
+          "dihip_gqa_attn")
+    return o
+
+
+def gqa_attn_mc_supported(ktable, vtable, G):
+    return bool(lib().dihip_gqa_attn_mc_supported(ktable.row_elems // G, vtable.row_elems // G, ktable.span_len, _DT[ktable.dtype]))
+
+
+def gqa_attn_mc(q, ktable, vtable, tok_pos, ent_slot, ent_row0, ent_count, max_count, max_pos, H, G, D, DV, scale, sink=None,
+                sink_mode=SINK_NONE, softcap=0.0, gate=None, out=None, nsplit=None):
+    """the matrix-core form (bf16 pages); max_count / max_pos: the largest portion and position of the step (host numbers)"""
+    T, E = q.shape[0], ent_slot.shape[0]
+    o = out if out is not None else torch.empty(T, H * DV, dtype=torch.float32, device=q.device)
+    if nsplit is None:       # fill the chip: ~2 workgroups per CU; at least 2 key tiles (64 keys) per workgroup
+        blocks = max(1, E * G * ((max_count * (H // G) + 63) // 64))
+        nsplit = max(1, min(512 // blocks, (max_pos + 1 + 63) // 64))
+    ws = None
+    if nsplit > 1:
+        ws = torch.empty(int(lib().dihip_gqa_attn_mc_workspace_bytes(T, H, DV, nsplit)), dtype=torch.uint8, device=q.device)
+    check(lib().dihip_gqa_attn_mc(stream(), ptr(o), _rows(o), ptr(q), _rows(q), ptr(ktable.ptrs), ptr(vtable.ptrs), ktable.max_spans,
+                                  ktable.span_len, ptr(sink), dt(sink) if sink is not None else F32_CODE, int(sink_mode), float(softcap or 0.0),
+                                  ptr(gate), _rows(gate) if gate is not None else 0, ptr(tok_pos), ptr(ent_slot), ptr(ent_row0), ptr(ent_count),
+                                  E, int(max_count), T, H, G, D, DV, float(scale), int(nsplit), ptr(ws), ws.numel() if ws is not None else 0),
+          "dihip_gqa_attn_mc")
+    return o
+
+
+CHUNKED_GLA_ROWS = 128   # portions from this length on run as chunks side by side
+
+
+def gla(q, k, v, z, q_scale, tau, state, ent_slot, ent_row0, ent_count, max_count, H, D, DV, out=None, chunked=None):
+    """q, k, z: f32 [T, >= H * D] rows, v: [T, >= H * DV]; state [slots, H, D, DV] f32 -> f32 [T, H * DV]"""
+    T, E = q.shape[0], ent_slot.shape[0]
+    assert state.shape[1:] == (H, D, DV) and state.is_contiguous()
+    o = out if out is not None else torch.empty(T, H * DV, dtype=torch.float32, device=q.device)
+    if chunked is None:
+        chunked = max_count >= CHUNKED_GLA_ROWS
+    ws = None
+    if chunked:
+        ws = torch.empty(int(lib().dihip_gla_chunked_workspace_bytes(E, int(max_count), H, D, DV)), dtype=torch.uint8, device=q.device)
+    check(lib().dihip_gla(stream(), ptr(o), _rows(o), ptr(q), _rows(q), ptr(k), _rows(k), ptr(v), _rows(v), ptr(z), _rows(z), float(q_scale),
+                          float(tau), ptr(state), ptr(ent_slot), ptr(ent_row0), ptr(ent_count), E, int(max_count), H, D, DV, 1 if chunked else 0,
+                          ptr(ws), ws.numel() if ws is not None else 0), "dihip_gla")
+    return o
+
+
+def head_rmsnorm_mul(x, gamma, eps, H, DV, mul=None, out=None):
+    T = x.shape[0]
+    y = out if out is not None else torch.empty(T, H * DV, dtype=torch.float32, device=x.device)
+    check(lib().dihip_head_rmsnorm_mul(stream(), ptr(y), dt(y), _rows(y), ptr(x), _rows(x), ptr(gamma), dt(gamma), float(eps), ptr(mul),
+                                       _rows(mul) if mul is not None else 0, T, H, DV), "dihip_head_rmsnorm_mul")
+    return y
+
+
+def moe_route(logits, top):
+    """-> ids [T, top] i32, wts [T, top] f32, seg [E + 1], src_row [T * top], dst [T * top]"""
+    T, E = logits.shape
+    dev = logits.device
+    ints = torch.empty(T * top * 3 + 2 * E + 1, dtype=torch.int32, device=dev)
+    ids, src_row, dst = ints[: T * top], ints[T * top: 2 * T * top], ints[2 * T * top: 3 * T * top]
+    counts, seg = ints[3 * T * top: 3 * T * top + E], ints[3 * T * top + E:]
+    wts = torch.empty(T, top, dtype=torch.float32, device=dev)
+    check(lib().dihip_seq_moe_route(stream(), ptr(logits), _rows(logits), ptr(ids), ptr(wts), ptr(counts), ptr(seg), ptr(src_row), ptr(dst),
+                                    T, E, int(top)), "dihip_seq_moe_route")
+    return ids.view(T, top), wts, seg, src_row, dst
+
+
+def moe_glu(gu, F, limit, slope, out):
+    R = gu.shape[0]
+    check(lib().dihip_seq_moe_glu(stream(), ptr(out), dt(out), _rows(out), ptr(gu), _rows(gu), R, F, float(limit), float(slope)),
+          "dihip_seq_moe_glu")
+    return out
+
+
+def moe_combine(rows, dst, wts, T, top, out=None):
+    K = rows.shape[1]
+    o = out if out is not None else torch.empty(T, K, dtype=torch.float32, device=rows.device)
+    check(lib().dihip_seq_moe_combine(stream(), ptr(o), _rows(o), ptr(rows), _rows(rows), ptr(dst), ptr(wts), T, int(top), K),
+          "dihip_seq_moe_combine")
     return o

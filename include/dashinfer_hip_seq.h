@@ -40,6 +40,78 @@ int dihip_linear(void* stream, const void* x, int x_dtype, long ldx, long x_gstr
                  const void* w, int w_dtype, const void* bias, void* y, int y_dtype, long ldy, long y_gstride,
                  const float* mul, long ldm, int T, int N, int K, int groups, int act, int act_lo, int act_hi, int math);
 
+/* The same product for rows that are grouped by owner (mixture of experts): group g owns the output rows seg[g] .. seg[g + 1]
+ * (seg: [groups + 1] on the device, ascending, seg[groups] <= R), output row r reads the x row row_map[r] (NULL: r itself) and
+ * the weight w[g] ([groups][N][K]); bias [groups][N] or NULL; `act` on every column.  seg_max_rows: a host-known bound on the
+ * rows of one group (it sizes the grid and chooses the kernel). */
+int dihip_linear_segmented(void* stream, const void* x, int x_dtype, long ldx, const void* w, int w_dtype, const void* bias,
+                           void* y, int y_dtype, long ldy, int R, int N, int K, int groups, const int32_t* seg,
+                           const int32_t* row_map, int seg_max_rows, int act, int math);
+
+/* The norm without statistics, fused with the residual step of a layer whose sublayers run side by side:
+ *   x_out[r] = x_in[r] + (a[r] + b[r])   (a NULL: x_in itself; b NULL: a alone),   h[i] = tanh(alpha * x_out[r]) * w + bias
+ * r = row_idx ? row_idx[i] : i (with row_idx x_out must be NULL).  x_in / x_out: contiguous [., K] f32 (may alias); h f32
+ * and / or h16 bf16 [M, K] (either may be NULL; w NULL: no norm). */
+int dihip_add_dyt(void* stream, float* x_out, const float* x_in, const float* a, long lda, const float* b, long ldb,
+                  const int32_t* row_idx, float alpha, const void* w, const void* bias, int w_dtype, float* h, void* h16,
+                  int M, int K);
+
+/* Grouped-query attention, step 1: per token the rows qkv[t] hold q [H, D] at column q_off, k [G, D] at k_off, v [G, DV] at
+ * v_off (f32).  Every query and key head is divided by its root mean square and scaled by qnorm / knorm [D] (NULL: no norm),
+ * then rotated on its first rot_dims dimensions by the angles tok_pos[t] * freq[i] (f32 product; layout 0: dimension 2i
+ * with 2i + 1, layout 1: i with i + rot_dims / 2; cos and sin times `mag`).  Queries are written back in place, keys go to
+ * the key pages (rows of G * D elements of cache_dtype), values to the value pages (rows of G * DV) after
+ *   v <- (1 - lam) v + lam vfirst_in[t]   (vfirst_in NULL: v as it is);   vfirst_out[t] <- v   (NULL: not kept). */
+int dihip_qkv_prep_append(void* stream, float* qkv, long ld, int q_off, int k_off, int v_off, int H, int G, int D, int DV,
+                          const void* qnorm, const void* knorm, int w_dtype, float eps, const float* freq, int rot_dims,
+                          int layout, float mag, float lam, const float* vfirst_in, float* vfirst_out, long ldvf,
+                          void* const* kspans, void* const* vspans, int span_stride, int span_len, int cache_dtype,
+                          const int32_t* tok_slot, const int32_t* tok_pos, int T);
+
+/* step 2: causal attention of every row over its sequence's pages; query head h reads key/value head h / (H / G):
+ *   s_j = scale * q[t, h] . k_j,  softcap > 0: s_j <- softcap * tanh(s_j / softcap),  j <= tok_pos[t]
+ *   p = softmax over {s_j} and, with sink_mode 1 / 2, one more logit sink[h] / 0 that has no value
+ *   out[t, h] = gate[t, h] * sum_j p_j v_j   (gate NULL: 1)
+ * q [T, H, D], out [T, H, DV] f32.  Every product and sum in f32. */
+int dihip_gqa_attn(void* stream, float* out, long ldo, const float* q, long ldq, void* const* kspans, void* const* vspans,
+                   int span_stride, int span_len, int cache_dtype, const void* sink, int w_dtype, int sink_mode, float softcap,
+                   const float* gate, long ldg, const int32_t* tok_slot, const int32_t* tok_pos, int T, int H, int G, int D,
+                   int DV, float scale);
+/* the same on the matrix cores for bf16 pages (D, DV multiples of 8 up to 256 / 128, span_len a multiple of 32): rows given
+ * as portions, the key walk split over nsplit workgroups (see dihip_latent_window_attn_mc) */
+int dihip_gqa_attn_mc_supported(int D, int DV, int span_len, int cache_dtype);
+size_t dihip_gqa_attn_mc_workspace_bytes(int T, int H, int DV, int nsplit);
+int dihip_gqa_attn_mc(void* stream, float* out, long ldo, const float* q, long ldq, void* const* kspans, void* const* vspans,
+                      int span_stride, int span_len, const void* sink, int w_dtype, int sink_mode, float softcap,
+                      const float* gate, long ldg, const int32_t* tok_pos, const int32_t* ent_slot, const int32_t* ent_row0,
+                      const int32_t* ent_count, int E, int max_count, int T, int H, int G, int D, int DV, float scale,
+                      int nsplit, void* ws, size_t ws_bytes);
+
+/* Gated linear attention, per head and portion, rows in order, f32:
+ *   alpha = sigmoid(z[t, h, :])^(1 / tau);   S <- diag(alpha) S + k[t, h] v[t, h]^T;   out[t, h] = S^T (q[t, h] * q_scale)
+ * S: state [slots][H][D][DV] f32, read at the portion's start and written back at its end.  chunked != 0: portions cut into
+ * chunks of 64 rows that run side by side (three launches, workspace .._workspace_bytes; f32 rounding differs). */
+size_t dihip_gla_chunked_workspace_bytes(int E, int max_count, int H, int D, int DV);
+int dihip_gla(void* stream, float* out, long ldo, const float* q, long ldq, const float* k, long ldk, const float* v, long ldv,
+              const float* z, long ldz, float q_scale, float tau, float* state, const int32_t* ent_slot,
+              const int32_t* ent_row0, const int32_t* ent_count, int E, int max_count, int H, int D, int DV, int chunked,
+              void* ws, size_t ws_bytes);
+/* y[t, h, :] = x[t, h, :] / sqrt(mean(x[t, h, :]^2) + eps) * gamma * mul[t, h, :]   (gamma [DV] shared by the heads; mul NULL: 1) */
+int dihip_head_rmsnorm_mul(void* stream, void* y, int y_dtype, long ldy, const float* x, long ldx, const void* gamma,
+                           int w_dtype, float eps, const float* mul, long ldm, int T, int H, int DV);
+
+/* Mixture of experts: per token the `top` experts of largest logit (ties: the lower index) and the softmax over the chosen
+ * logits -> ids / wts [T, top]; the T * top (token, choice) pairs grouped by expert -> seg [E + 1], src_row [T * top] (the
+ * token a sorted row reads), dst [T * top] (the sorted row of pair t * top + k); counts: [E] scratch. */
+int dihip_seq_moe_route(void* stream, const float* logits, long ldl, int32_t* ids, float* wts, int32_t* counts, int32_t* seg,
+                    int32_t* src_row, int32_t* dst, int T, int E, int top);
+/* y[r, c] = g * sigmoid(slope * g) * (u + 1),  g = min(gu[r, c], limit),  u = clamp(gu[r, F + c], -limit, limit) */
+int dihip_seq_moe_glu(void* stream, void* y, int y_dtype, long ldy, const float* gu, long ldgu, int R, int F, float limit,
+                  float slope);
+/* out[t] = sum_k wts[t, k] * rows[dst[t * top + k]],  k ascending */
+int dihip_seq_moe_combine(void* stream, float* out, long ldo, const float* rows, long ldr, const int32_t* dst, const float* wts,
+                      int T, int top, int K);
+
 /* h[t, :] = float(table[ids[t], :]) + float(table2[rows2[t], :])   (table2 NULL: the first term alone) */
 int dihip_embed_sum(void* stream, float* h, const int32_t* ids, const void* table, const int32_t* rows2,
                     const void* table2, int w_dtype, int T, int K);
