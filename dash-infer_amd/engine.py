@@ -94,7 +94,9 @@ class SeqEngine:
             return self._decode_step(host, cut, T, max(tpos))
         if torch.cuda.is_available():
             host = host.pin_memory()
-        ctx = self._context(host.to(self.device, non_blocking=True), cut, T, E, max(ecnt), max(tpos))
+        # the split of the attention's key walk follows the length bucket, as in the captured decode steps: the same step gives the
+        # same bits whether it is launched or replayed
+        ctx = self._context(host.to(self.device, non_blocking=True), cut, T, E, max(ecnt), self._bucket(max(tpos)))
         ctx.taps = taps
         x = model.forward(ctx)
         if not want:
@@ -110,10 +112,15 @@ class SeqEngine:
         ctx.max_count, ctx.max_pos = max_count, max_pos
         return ctx
 
+    @staticmethod
+    def _bucket(max_pos):
+        """the last position of the 512-position bucket max_pos lies in: the split of the attention's key walk follows this, not the exact length"""
+        return (max_pos + 512) // 512 * 512 - 1
+
     def _decode_step(self, host, cut, E, max_pos):
         """one token of each of E requests: the first step of a (E, length bucket) runs eagerly and is then captured, later ones
         replay.  The returned logits are the graph's own buffer: valid until the next step."""
-        bucket = (max_pos + 512) // 512 * 512 - 1       # the split of the attention's key walk follows this, not the exact length
+        bucket = self._bucket(max_pos)
         g = self._graphs.get((E, bucket))
         if g is None:
             g = {"host": torch.empty(host.numel(), dtype=torch.int32, pin_memory=True),
