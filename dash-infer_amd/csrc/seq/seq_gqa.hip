@@ -24,8 +24,15 @@ struct PrepArgs {
 
 __global__ __launch_bounds__(256) void qkv_prep_append_kernel(PrepArgs a) {
   __shared__ float hs[4][256];
+  __shared__ float cs_t[128], sn_t[128];   // the token's cos and sin per rotated pair, shared by all heads
   const int t = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int pos = a.tok_pos[t];
+  if (threadIdx.x < (a.rot_dims >> 1)) {
+    float sn, cs;
+    rope_sincos((uint32_t)pos, a.freq[threadIdx.x], &sn, &cs);
+    cs_t[threadIdx.x] = cs * a.mag;
+    sn_t[threadIdx.x] = sn * a.mag;
+  }
   const size_t sp = (size_t)a.tok_slot[t] * a.span_stride + pos / a.span_len;
   const size_t in_span = (size_t)(pos % a.span_len);
   float* row = a.qkv + (size_t)t * a.ld;
@@ -67,9 +74,7 @@ __global__ __launch_bounds__(256) void qkv_prep_append_kernel(PrepArgs a) {
           bool first;
           if (a.layout == 0) { pair = d >> 1; first = (d & 1) == 0; other = d ^ 1; }
           else { first = d < half; pair = first ? d : d - half; other = first ? d + half : d - half; }
-          float sn, cs;
-          rope_sincos((uint32_t)pos, a.freq[pair], &sn, &cs);
-          sn *= a.mag; cs *= a.mag;
+          const float sn = sn_t[pair], cs = cs_t[pair];
           const float o = hs[wave][other];
           y = first ? v[i] * cs - o * sn : v[i] * cs + o * sn;
         }

@@ -254,12 +254,11 @@ def gla(q, k, v, z, q_scale, tau, state, ent_slot, ent_row0, ent_count, max_coun
     o = out if out is not None else torch.empty(T, H * DV, dtype=torch.float32, device=q.device)
     if chunked is None:
         chunked = max_count >= CHUNKED_GLA_ROWS
-    ws = None
-    if chunked:
-        ws = torch.empty(int(lib().dihip_gla_chunked_workspace_bytes(E, int(max_count), H, D, DV)), dtype=torch.uint8, device=q.device)
+    chunked = 1 if chunked else 0
+    ws = torch.empty(int(lib().dihip_gla_workspace_bytes(T, E, int(max_count), H, D, DV, chunked)), dtype=torch.uint8, device=q.device)
     check(lib().dihip_gla(stream(), ptr(o), _rows(o), ptr(q), _rows(q), ptr(k), _rows(k), ptr(v), _rows(v), ptr(z), _rows(z), float(q_scale),
-                          float(tau), ptr(state), ptr(ent_slot), ptr(ent_row0), ptr(ent_count), E, int(max_count), H, D, DV, 1 if chunked else 0,
-                          ptr(ws), ws.numel() if ws is not None else 0), "dihip_gla")
+                          float(tau), ptr(state), ptr(ent_slot), ptr(ent_row0), ptr(ent_count), T, E, int(max_count), H, D, DV, chunked,
+                          ptr(ws), ws.numel()), "dihip_gla")
     return o
 
 

@@ -90,12 +90,13 @@ int dihip_gqa_attn_mc(void* stream, float* out, long ldo, const float* q, long l
 /* Gated linear attention, per head and portion, rows in order, f32:
  *   alpha = sigmoid(z[t, h, :])^(1 / tau);   S <- diag(alpha) S + k[t, h] v[t, h]^T;   out[t, h] = S^T (q[t, h] * q_scale)
  * S: state [slots][H][D][DV] f32, read at the portion's start and written back at its end.  chunked != 0: portions cut into
- * chunks of 64 rows that run side by side (three launches, workspace .._workspace_bytes; f32 rounding differs). */
-size_t dihip_gla_chunked_workspace_bytes(int E, int max_count, int H, int D, int DV);
+ * chunks of 64 rows that run side by side (f32 rounding differs).  ws: .._workspace_bytes, always needed (the rows' decays,
+ * keys and scaled queries are staged there). */
+size_t dihip_gla_workspace_bytes(int T, int E, int max_count, int H, int D, int DV, int chunked);
 int dihip_gla(void* stream, float* out, long ldo, const float* q, long ldq, const float* k, long ldk, const float* v, long ldv,
               const float* z, long ldz, float q_scale, float tau, float* state, const int32_t* ent_slot,
-              const int32_t* ent_row0, const int32_t* ent_count, int E, int max_count, int H, int D, int DV, int chunked,
-              void* ws, size_t ws_bytes);
+              const int32_t* ent_row0, const int32_t* ent_count, int T, int E, int max_count, int H, int D, int DV,
+              int chunked, void* ws, size_t ws_bytes);
 /* y[t, h, :] = x[t, h, :] / sqrt(mean(x[t, h, :]^2) + eps) * gamma * mul[t, h, :]   (gamma [DV] shared by the heads; mul NULL: 1) */
 int dihip_head_rmsnorm_mul(void* stream, void* y, int y_dtype, long ldy, const float* x, long ldx, const void* gamma,
                            int w_dtype, float eps, const float* mul, long ldm, int T, int H, int DV);
