@@ -195,7 +195,7 @@ __global__ __launch_bounds__(256) void head_rmsnorm_mul_kernel(void* __restrict_
                                                                const void* __restrict__ gamma, float eps, const float* __restrict__ mul,
                                                                long ldm, int H, int DV) {
   const int t = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  for (int h = wave; h < H; h += 4) {
+  for (int h = blockIdx.y * 4 + wave; h < H; h += 4 * gridDim.y) {
     const float* xr = x + (size_t)t * ldx + (size_t)h * DV;
     float ss = 0.f;
     for (int d = lane; d < DV; d += 64) ss = __builtin_fmaf(xr[d], xr[d], ss);
@@ -271,8 +271,9 @@ int dihip_head_rmsnorm_mul(void* stream, void* y, int y_dtype, long ldy, const f
                     seq_dtype_ok(y_dtype) && seq_dtype_ok(w_dtype), DIHIP_PARAM_ERROR, "head_rmsnorm_mul: bad argument");
   if (T == 0) return DIHIP_SUCCESS;
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
-  if (w_dtype == DIHIP_F32) hipLaunchKernelGGL(head_rmsnorm_mul_kernel<DIHIP_F32>, dim3(T), dim3(256), 0, s, y, y_dtype, ldy, x, ldx, gamma, eps, mul, ldm, H, DV);
-  else hipLaunchKernelGGL(head_rmsnorm_mul_kernel<DIHIP_BF16>, dim3(T), dim3(256), 0, s, y, y_dtype, ldy, x, ldx, gamma, eps, mul, ldm, H, DV);
+  const dim3 grid(T, T >= 256 ? 1 : (H + 3) / 4);   // few rows (decoding): a wave per head; many rows: a workgroup per row
+  if (w_dtype == DIHIP_F32) hipLaunchKernelGGL(head_rmsnorm_mul_kernel<DIHIP_F32>, grid, dim3(256), 0, s, y, y_dtype, ldy, x, ldx, gamma, eps, mul, ldm, H, DV);
+  else hipLaunchKernelGGL(head_rmsnorm_mul_kernel<DIHIP_BF16>, grid, dim3(256), 0, s, y, y_dtype, ldy, x, ldx, gamma, eps, mul, ldm, H, DV);
   return launch_status();
 }
 

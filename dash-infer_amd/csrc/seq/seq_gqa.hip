@@ -37,7 +37,7 @@ __global__ __launch_bounds__(256) void qkv_prep_append_kernel(PrepArgs a) {
   const size_t in_span = (size_t)(pos % a.span_len);
   float* row = a.qkv + (size_t)t * a.ld;
   const int D = a.D, half = a.rot_dims >> 1;
-  for (int h0 = 0; h0 < a.H + a.G; h0 += 4) {      // query heads, then key heads: the same trip count in every wave
+  for (int h0 = blockIdx.y * 4; h0 < a.H + a.G; h0 += 4 * gridDim.y) {      // query heads, then key heads: the same trip count in every wave
     const int hh = h0 + wave;
     const bool live = hh < a.H + a.G, is_q = hh < a.H;
     float* src = row + (is_q ? a.q_off + hh * D : a.k_off + (hh - a.H) * D);
@@ -85,7 +85,7 @@ __global__ __launch_bounds__(256) void qkv_prep_append_kernel(PrepArgs a) {
   }
   void* vdst = a.vspans[sp];
   const int nv = a.G * a.DV;
-  for (int e = threadIdx.x; e < nv; e += 256) {
+  for (int e = blockIdx.y * 256 + threadIdx.x; e < nv; e += 256 * gridDim.y) {
     float v = row[a.v_off + e];
     if (a.vfirst_in) v = (1.f - a.lam) * v + a.lam * a.vfirst_in[(size_t)t * a.ldvf + e];
     if (a.vfirst_out) a.vfirst_out[(size_t)t * a.ldvf + e] = v;
@@ -431,7 +431,8 @@ int dihip_qkv_prep_append(void* stream, float* qkv, long ld, int q_off, int k_of
   if (T == 0) return DIHIP_SUCCESS;
   PrepArgs a{qkv, ld, q_off, k_off, v_off, H, G, D, DV, qnorm, knorm, w_dtype, eps, freq, rot_dims, layout, mag, lam, vfirst_in, vfirst_out,
              ldvf, kspans, vspans, span_stride, span_len, cache_dtype, tok_slot, tok_pos};
-  hipLaunchKernelGGL(qkv_prep_append_kernel, dim3(T), dim3(256), 0, reinterpret_cast<hipStream_t>(stream), a);
+  // few rows (decoding): the heads of a token are spread over workgroups of four; many rows: a workgroup per token
+  hipLaunchKernelGGL(qkv_prep_append_kernel, dim3(T, T >= 256 ? 1 : (H + G + 3) / 4), dim3(256), 0, reinterpret_cast<hipStream_t>(stream), a);
   return launch_status();
 }
 

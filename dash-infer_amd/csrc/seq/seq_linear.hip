@@ -313,6 +313,35 @@ __global__ __launch_bounds__(256) void linear_skinny_kernel(LinArgs a, int t0, i
     }
 }
 
+// Few output columns against many rows (a router's logits): one workgroup per row, the row staged in LDS as f32, a wave per
+// column: f32 products of the unrounded row, each lane over its k in ascending order, then the fixed tree over the lanes.
+// K % 8 == 0 and 16-byte aligned weight rows (host-checked).
+template <int XT>
+__global__ __launch_bounds__(256) void linear_fewcols_kernel(LinArgs a) {
+  extern __shared__ __attribute__((aligned(16))) float xrow[];
+  const int t = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  for (int k = tid; k < a.K; k += 256) xrow[k] = load_ft<XT>(a.x, (size_t)t * a.ldx + k);
+  __syncthreads();
+  for (int n = wave; n < a.N; n += 4) {
+    const uint16_t* wr = (const uint16_t*)a.w + (size_t)n * a.K;
+    float acc = 0.f;
+    for (int k = lane * 8; k < a.K; k += 512) {
+      const u32x4_t wv = *reinterpret_cast<const u32x4_t*>(wr + k);
+      const f32x4_t lo = *reinterpret_cast<const f32x4_t*>(xrow + k), hi = *reinterpret_cast<const f32x4_t*>(xrow + k + 4);
+      acc = __builtin_fmaf(__uint_as_float(wv[0] << 16), lo[0], acc);
+      acc = __builtin_fmaf(__uint_as_float(wv[0] & 0xffff0000u), lo[1], acc);
+      acc = __builtin_fmaf(__uint_as_float(wv[1] << 16), lo[2], acc);
+      acc = __builtin_fmaf(__uint_as_float(wv[1] & 0xffff0000u), lo[3], acc);
+      acc = __builtin_fmaf(__uint_as_float(wv[2] << 16), hi[0], acc);
+      acc = __builtin_fmaf(__uint_as_float(wv[2] & 0xffff0000u), hi[1], acc);
+      acc = __builtin_fmaf(__uint_as_float(wv[3] << 16), hi[2], acc);
+      acc = __builtin_fmaf(__uint_as_float(wv[3] & 0xffff0000u), hi[3], acc);
+    }
+    acc = wave_sum(acc);
+    if (lane == 0) lin_epilogue(a, 0, t, n, acc, DIHIP_BF16);
+  }
+}
+
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 }  // namespace
@@ -349,6 +378,11 @@ static int linear_impl(void* stream, const void* x, int x_dtype, long ldx, long 
         if (x_dtype == DIHIP_F32) hipLaunchKernelGGL((linear_skinny_kernel<DIHIP_F32, true>), grid, dim3(256), (size_t)tc * K * 4, s, a, t0, tc);
         else hipLaunchKernelGGL((linear_skinny_kernel<DIHIP_BF16, true>), grid, dim3(256), (size_t)tc * K * 4, s, a, t0, tc);
       }
+      return launch_status();
+    }
+    if (N <= 64 && groups == 1 && !seg && vec && K <= 16384) {   // many rows, few columns: the tile kernel would idle most of its 64 x 64 tile
+      if (x_dtype == DIHIP_F32) hipLaunchKernelGGL((linear_fewcols_kernel<DIHIP_F32>), dim3(T), dim3(256), (size_t)K * 4, s, a);
+      else hipLaunchKernelGGL((linear_fewcols_kernel<DIHIP_BF16>), dim3(T), dim3(256), (size_t)K * 4, s, a);
       return launch_status();
     }
     math = DIHIP_MATH_F32;

@@ -129,8 +129,9 @@ __global__ __launch_bounds__(256) void add_dyt_kernel(float* x_out, const float*
                                                       uint16_t* __restrict__ h16, int K) {
   const int i = blockIdx.x;
   const size_t r = row_idx ? (size_t)row_idx[i] : (size_t)i;
+  const int k_lo = blockIdx.y * 1024, k_hi = min(K, k_lo + 1024);   // a row's columns are spread over gridDim.y workgroups (few rows: decoding)
 #pragma unroll 4
-  for (int k = threadIdx.x; k < K; k += 256) {
+  for (int k = k_lo + threadIdx.x; k < k_hi; k += 256) {
     float v = x_in[r * K + k];
     if (a) {
       float s = a[r * lda + k];
@@ -439,8 +440,8 @@ int dihip_add_dyt(void* stream, float* x_out, const float* x_in, const float* a,
                     seq_dtype_ok(w_dtype), DIHIP_PARAM_ERROR, "add_dyt: bad argument");
   if (M == 0) return DIHIP_SUCCESS;
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
-  if (w_dtype == DIHIP_F32) hipLaunchKernelGGL(add_dyt_kernel<DIHIP_F32>, dim3(M), dim3(256), 0, s, x_out, x_in, a, lda, b, ldb, row_idx, alpha, w, bias, h, (uint16_t*)h16, K);
-  else hipLaunchKernelGGL(add_dyt_kernel<DIHIP_BF16>, dim3(M), dim3(256), 0, s, x_out, x_in, a, lda, b, ldb, row_idx, alpha, w, bias, h, (uint16_t*)h16, K);
+  if (w_dtype == DIHIP_F32) hipLaunchKernelGGL(add_dyt_kernel<DIHIP_F32>, dim3(M, (K + 1023) / 1024), dim3(256), 0, s, x_out, x_in, a, lda, b, ldb, row_idx, alpha, w, bias, h, (uint16_t*)h16, K);
+  else hipLaunchKernelGGL(add_dyt_kernel<DIHIP_BF16>, dim3(M, (K + 1023) / 1024), dim3(256), 0, s, x_out, x_in, a, lda, b, ldb, row_idx, alpha, w, bias, h, (uint16_t*)h16, K);
   return launch_status();
 }
 

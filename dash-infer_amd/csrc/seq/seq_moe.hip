@@ -15,8 +15,8 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict_
   const int t = blockIdx.x * 256 + threadIdx.x;
   if (t >= T) return;
   const float* z = logits + (size_t)t * ldl;
-  float best[16];
-  int bi[16];
+  float best[32];
+  int bi[32];
   for (int k = 0; k < top; ++k) {
     float bv = -INFINITY;
     int bx = -1;
@@ -79,7 +79,7 @@ __global__ __launch_bounds__(256) void moe_place_kernel(const int32_t* __restric
 __global__ __launch_bounds__(256) void moe_glu_kernel(void* __restrict__ y, int ydt, long ldy, const float* __restrict__ gu, long ldgu, int F,
                                                       float limit, float slope) {
   const int r = blockIdx.x;
-  for (int c = threadIdx.x; c < F; c += 256) {
+  for (int c = blockIdx.y * 256 + threadIdx.x; c < F; c += 256 * gridDim.y) {
     const float g = fminf(gu[(size_t)r * ldgu + c], limit);
     const float u = fminf(fmaxf(gu[(size_t)r * ldgu + F + c], -limit), limit);
     st_any(y, (size_t)r * ldy + c, ydt, g * (1.f / (1.f + expf(-slope * g))) * (u + 1.f));
@@ -89,7 +89,7 @@ __global__ __launch_bounds__(256) void moe_glu_kernel(void* __restrict__ y, int 
 __global__ __launch_bounds__(256) void moe_combine_kernel(float* __restrict__ out, long ldo, const float* __restrict__ rows, long ldr,
                                                           const int32_t* __restrict__ dst, const float* __restrict__ wts, int top, int K) {
   const int t = blockIdx.x;
-  for (int c = threadIdx.x; c < K; c += 256) {
+  for (int c = blockIdx.y * 256 + threadIdx.x; c < K; c += 256 * gridDim.y) {
     float acc = 0.f;
     for (int k = 0; k < top; ++k) acc = __builtin_fmaf(wts[(size_t)t * top + k], rows[(size_t)dst[(size_t)t * top + k] * ldr + c], acc);
     out[(size_t)t * ldo + c] = acc;
@@ -105,8 +105,8 @@ extern "C" {
 
 int dihip_seq_moe_route(void* stream, const float* logits, long ldl, int32_t* ids, float* wts, int32_t* counts, int32_t* seg, int32_t* src_row,
                     int32_t* dst, int T, int E, int top) {
-  DIHIP_REQUIRE(T >= 0 && E > 0 && top > 0 && top <= E && top <= 16 && E <= 65535 && logits && ids && wts && counts && seg && src_row && dst &&
-                    ldl >= E, DIHIP_PARAM_ERROR, "moe_route: bad argument (at most 16 choices per token)");
+  DIHIP_REQUIRE(T >= 0 && E > 0 && top > 0 && top <= E && top <= 32 && E <= 65535 && logits && ids && wts && counts && seg && src_row && dst &&
+                    ldl >= E, DIHIP_PARAM_ERROR, "moe_route: bad argument (at most 32 choices per token)");
   if (T == 0) return DIHIP_SUCCESS;
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
   hipLaunchKernelGGL(moe_route_kernel, dim3((T + 255) / 256), dim3(256), 0, s, logits, ldl, ids, wts, T, E, top);
@@ -118,7 +118,7 @@ int dihip_seq_moe_route(void* stream, const float* logits, long ldl, int32_t* id
 int dihip_seq_moe_glu(void* stream, void* y, int y_dtype, long ldy, const float* gu, long ldgu, int R, int F, float limit, float slope) {
   DIHIP_REQUIRE(R >= 0 && F > 0 && y && gu && ldy >= F && ldgu >= 2 * (long)F && seq_dtype_ok(y_dtype), DIHIP_PARAM_ERROR, "moe_glu: bad argument");
   if (R == 0) return DIHIP_SUCCESS;
-  hipLaunchKernelGGL(moe_glu_kernel, dim3(R), dim3(256), 0, reinterpret_cast<hipStream_t>(stream), y, y_dtype, ldy, gu, ldgu, F, limit, slope);
+  hipLaunchKernelGGL(moe_glu_kernel, dim3(R, R >= 256 ? 1 : (F + 1023) / 1024), dim3(256), 0, reinterpret_cast<hipStream_t>(stream), y, y_dtype, ldy, gu, ldgu, F, limit, slope);
   return launch_status();
 }
 
@@ -126,7 +126,7 @@ int dihip_seq_moe_combine(void* stream, float* out, long ldo, const float* rows,
                       int K) {
   DIHIP_REQUIRE(T >= 0 && top > 0 && K > 0 && out && rows && dst && wts && ldo >= K && ldr >= K, DIHIP_PARAM_ERROR, "moe_combine: bad argument");
   if (T == 0) return DIHIP_SUCCESS;
-  hipLaunchKernelGGL(moe_combine_kernel, dim3(T), dim3(256), 0, reinterpret_cast<hipStream_t>(stream), out, ldo, rows, ldr, dst, wts, top, K);
+  hipLaunchKernelGGL(moe_combine_kernel, dim3(T, T >= 256 ? 1 : (K + 1023) / 1024), dim3(256), 0, reinterpret_cast<hipStream_t>(stream), out, ldo, rows, ldr, dst, wts, top, K);
   return launch_status();
 }
 

@@ -287,3 +287,19 @@ def test_routed_experts(so, experts, top, T):
     assert rel_err(rig16.step([("a", h)])[0], want) < 0.03
     if T > 1:                                                     # a token's result does not depend on the others of the batch
         assert rel_err(rig.step([("b", h[T // 2:T // 2 + 1])])[0], got[T // 2:T // 2 + 1]) < 1e-6
+
+
+@pytest.mark.parametrize("T,N,K", [(100, 12, 192), (300, 5, 64), (40, 64, 1000), (17, 1, 8)])
+def test_router_logits_many_rows_few_columns(so, T, N, K):
+    """the f32 product of many rows with few output columns: unrounded operands, the same bits for a row whatever the batch"""
+    rng = np.random.default_rng(T + N)
+    x = rng.normal(0, 1, (T, K)).astype(np.float32)
+    w, b = bf(rng.normal(0, 0.3, (N, K))), bf(rng.normal(0, 0.3, N))
+    want = x.astype(np.float64) @ w.astype(np.float64).T + b
+    got = so.linear(dev(x), dev(w, torch.bfloat16), dev(b, torch.bfloat16), math=so.MATH_F32_STREAM)
+    assert rel_err(got.cpu().numpy(), want) < 2e-6
+    part = so.linear(dev(x[T // 2:T // 2 + 20]), dev(w, torch.bfloat16), dev(b, torch.bfloat16), math=so.MATH_F32_STREAM)
+    assert torch.equal(part.cpu(), got.cpu()[T // 2:T // 2 + 20])
+    x16 = dev(x, torch.bfloat16)
+    got16 = so.linear(x16, dev(w, torch.bfloat16), dev(b, torch.bfloat16), math=so.MATH_F32_STREAM)
+    assert rel_err(got16.cpu().numpy(), x16.double().cpu().numpy() @ w.astype(np.float64).T + b) < 2e-6
