@@ -80,6 +80,7 @@ SHAPES = [  # width, heads, kv heads, dim, vdim, rotated dims
     (80, 5, 1, 40, 8, 40),       # one key/value head, an odd number of query heads
     (64, 2, 1, 128, 64, 64),     # wide heads
     (48, 3, 3, 20, 12, 8),       # head sizes the matrix-core kernel does not serve
+    (64, 2, 1, 160, 128, 32),    # the widest tiles of the matrix-core kernel
 ]
 
 
@@ -206,7 +207,8 @@ def gla_rig(w, m, dtype, **kw):
     return MixerRig(lambda state, dt: mixers.GatedLinearAttention("t", m["heads"], m["dim"], m["vdim"], m["tau"], dev_weights(w), state), dtype, **kw)
 
 
-@pytest.mark.parametrize("shape", [(72, 3, 20, 24, 8, 8.0), (64, 1, 64, 64, 4, 1.0), (96, 2, 72, 130, 16, 12.0), (64, 2, 8, 200, 1, 2.0)])
+@pytest.mark.parametrize("shape", [(72, 3, 20, 24, 8, 8.0), (64, 1, 64, 64, 4, 1.0), (96, 2, 72, 130, 16, 12.0), (64, 2, 8, 200, 1, 2.0),
+                                   (64, 1, 136, 40, 4, 4.0)])
 def test_gla_whole_decoded_portions_and_chunks(shape):
     width, H, D, V, rank, tau = shape
     rng = np.random.default_rng(D + V)
